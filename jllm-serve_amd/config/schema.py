@@ -70,10 +70,11 @@ class NormSpec:
 @dataclass(frozen=True)
 class LayerNormSpec:
     """Layer norm with a weight and a bias: (x - mean) / sqrt(mean of squared deviations + eps) * w + b. The bias is the
-    tensor whose name is the weight's with ``bias_suffix`` added."""
+    tensor whose name is the weight's with ``bias_suffix`` added; ``bias`` False: the norm has a weight only."""
 
     eps: float
     bias_suffix: str = ".b"
+    bias: bool = True
     kind: str = "layernorm"
 
 
@@ -136,6 +137,7 @@ class GqaSpec:
 class LatentAttentionNames:
     """Tensor names of a latent-attention mixer under the layer's prefix (no ending: the tensors are named bare)."""
 
+    q: str = "mix.q"  # the query projection of a mixer without a query latent
     dq: str = "mix.dq"
     dq_norm: str = "mix.dq.norm"
     uq: str = "mix.uq"
@@ -155,7 +157,8 @@ class LatentAttentionSpec:
 
     Per position the layer caches the RMS-normed latent c (``kv_rank`` numbers) and one rotated key part of
     ``rot_dim`` numbers that all heads share; head h's unrotated key is W_uk[h] c and its value W_uv[h] c. A head's
-    query has ``dim`` unrotated and ``rot_dim`` rotated entries and comes from a normed latent of ``q_rank``.
+    query has ``dim`` unrotated and ``rot_dim`` rotated entries and comes from a normed latent of ``q_rank``
+    (``q_rank`` 0: straight from the input, by one projection ``q``).
     ``window`` 0 = all earlier keys, else the query at p sees keys p + 1 - window .. p. ``sink``: a learned number
     per head whose exponential joins the softmax's denominator. ``out_gate``: the concatenated heads are multiplied
     by sigmoid(W_g h) before the output product. ``owns_cache`` False: the run reads the cache of an earlier run (the
@@ -246,6 +249,11 @@ class GatedDeltaNames:
     gate: str = "g"
     o: str = "o"
     conv_suffix: str = ".conv"
+    # a decay or gate input that passes a narrow middle: W_up (W_down h)
+    decay_down: str = "a1"
+    decay_up: str = "a2"
+    gate_down: str = "g1"
+    gate_up: str = "g2"
 
 
 @dataclass(frozen=True)
@@ -255,7 +263,12 @@ class GatedDeltaSpec:
     h / (heads / kv_heads)), v has ``heads`` heads of ``vdim``; q, k and v pass a causal convolution of ``conv`` taps per
     channel and silu; q and k are made unit vectors (q also times dim^-1/2); the write strength is sigmoid(W_b h), the
     decay exp(-exp(A_log) softplus(W_a h + dt_bias)) per head; each head's read-out is divided by its root mean square
-    (``eps``), multiplied by a gain shared by the heads and by silu(W_g h), and goes through W_o."""
+    (``eps``), multiplied by a gain shared by the heads and by silu(W_g h), and goes through W_o.
+
+    ``decay`` "channel": one decay per head and key channel instead, g = exp(-exp(A_log_h) softplus(a + dt_bias)) with a
+    and dt_bias laid out heads x dim, acting on the rows of S that belong to the key channels. ``decay_rank`` > 0: the
+    decay's input is W_up (W_down h) through a middle of that many numbers (else one projection). ``gate_rank`` > 0: the
+    same for the output gate's input. ``gate_fn``: "silu" or "sigmoid"."""
 
     heads: int
     kv_heads: int
@@ -264,7 +277,45 @@ class GatedDeltaSpec:
     conv: int
     eps: float
     names: GatedDeltaNames = GatedDeltaNames()
+    decay: str = "head"
+    decay_rank: int = 0
+    gate_rank: int = 0
+    gate_fn: str = "silu"
     kind: str = "gated_delta"
+
+
+@dataclass(frozen=True)
+class StateSpaceNames:
+    """Tensor names of a state-space mixer under its prefix."""
+
+    in_proj: str = "in"
+    conv: str = "conv"
+    conv_bias: str = "conv.b"
+    dt_bias: str = "dt_bias"
+    a_log: str = "A_log"
+    skip: str = "D"
+    norm: str = "norm"
+    o: str = "o"
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A selective state-space mixer (the Mamba-2 form). One input projection gives [z | x | B | C | dt] with z and x
+    of heads x ``vdim``, B and C of ``groups`` x ``state`` and one dt per head; x, B and C together pass a causal
+    convolution of ``conv`` taps per channel with a bias, and silu. Per head (head h uses group h / (heads / groups)):
+    dt = softplus(dt + dt_bias), S <- exp(-exp(A_log) dt) S + dt B x^T with S [state, vdim], y = S^T C + D x. The
+    heads' y times silu(z) is RMS-normed in ``norm_groups`` equal parts (``eps``), multiplied by a weight, and goes
+    through W_o."""
+
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    norm_groups: int
+    conv: int
+    eps: float
+    names: StateSpaceNames = StateSpaceNames()
+    kind: str = "state_space"
 
 
 @dataclass(frozen=True)
@@ -336,6 +387,40 @@ class TableMoeSpec:
     kind: str = "table_moe"
 
 
+@dataclass(frozen=True)
+class RoutedMoeNames:
+    """Tensor names of a router-chosen mixture of experts under the layer's prefix: expert e's tensors are
+    ``<expert>{e}.<gate|up|down>``, the router's weight ``router`` and the choice scores' correction ``correction``."""
+
+    expert: str = "mlp.e"
+    gate: str = "gate"
+    up: str = "up"
+    down: str = "down"
+    router: str = "mlp.router"
+    correction: str = "mlp.correction"
+    ending: str = ""
+
+
+@dataclass(frozen=True)
+class RoutedMoeSpec:
+    """A mixture of small gated feed-forwards chosen by a router: scores s = sigmoid(W_router h) in fp32; the choice
+    scores are s + correction (``correction`` False: s alone); the experts form ``groups`` equal groups of neighbours, a
+    group's score is the sum of its two largest choice scores, and only experts of the ``keep`` best groups can be
+    chosen; the ``top`` largest choice scores win; their weights are their s divided by the sum (+ 1e-20) times
+    ``scale``. Experts are gated feed-forwards of ``hidden`` with the gate function ``activation``."""
+
+    experts: int
+    top: int
+    hidden: int
+    scale: float = 1.0
+    groups: int = 1
+    keep: int = 1
+    correction: bool = True
+    activation: str = "silu"
+    names: RoutedMoeNames = RoutedMoeNames()
+    kind: str = "routed_moe"
+
+
 # --------------------------------------------------------------------------- layers and model
 
 
@@ -344,7 +429,8 @@ class LayerSpec:
     """One decoder layer: which mixer, which feed-forward, which norms, and how they are arranged.
 
     ``arrangement`` "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) (model/LayerSpec.java:18-19,
-    cpu/CpuBackend.java:959-969). ``ffn`` None: the layer has no feed-forward (and no second norm). ``prefix`` is the tensor-name prefix of the layer's weights; the names under it
+    cpu/CpuBackend.java:959-969). "parallel": with h = norm(x), x += mixer(h) + ffn(h): one norm, both sublayers read it.
+    ``ffn`` None: the layer has no feed-forward (and no second norm). ``prefix`` is the tensor-name prefix of the layer's weights; the names under it
     are data of the specs (here the two norms', in the mixer's and feed-forward's specs theirs), so a checkpoint
     that names or stacks its tensors differently is a matter of the parser.
     """
@@ -374,15 +460,25 @@ class StreamVector:
 
 
 @dataclass(frozen=True)
+class StreamMix:
+    """The stream is replaced by W [x; x0] right before a run: x the stream, x0 the embedding output of the same rows,
+    W the tensor ``name`` [hidden, 2 hidden] with the stream's columns first."""
+
+    name: str
+
+
+@dataclass(frozen=True)
 class ScheduleEntry:
     """One step of the layer schedule: run ``layer``; ``cache_from`` names an earlier schedule entry
     whose cache this run reads instead of writing one of its own (None = its own cache); ``add_before``: a vector
     that joins the stream right before this run (a layer that runs several times with one set of weights has a cache
-    or state per run, and may be told which pass it is in this way)."""
+    or state per run, and may be told which pass it is in this way); ``mix_before``: the stream is first mixed with the
+    embedding output (before the vector joins)."""
 
     layer: int
     cache_from: Optional[int] = None
     add_before: Optional[StreamVector] = None
+    mix_before: Optional[StreamMix] = None
 
 
 @dataclass(frozen=True)
@@ -411,6 +507,7 @@ class ModelConfig:
     eos_token_ids: Tuple[int, ...] = ()
     max_positions: int = 4096
     embed_scale: float = 1.0
+    logit_scale: float = 1.0  # the logits are the head's product times this
     description: str = ""
     names: ModelNames = ModelNames()
     raw: Mapping[str, Any] = field(default_factory=dict, compare=False, repr=False)

@@ -161,3 +161,22 @@ extern "C" int jllm_copy_words(const void* src, void* dst, long long n_words, hi
   JLLM_CHECK_LAUNCH("copy_words");
   return 0;
 }
+
+// out[t] = [a[t] | b[t]] in out's type: two fp32 row sets (the stream and a second stream of the same width) side by
+// side as the input rows of one product.
+template <typename TO>
+__global__ __launch_bounds__(256) void concat_rows_kernel(const float* __restrict__ a, const float* __restrict__ b, int d,
+                                                         TO* __restrict__ out, int ldo) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < 2 * d; i += 256)
+    stf(out + (size_t)t * ldo, i, i < d ? a[(size_t)t * d + i] : b[(size_t)t * d + i - d]);
+}
+
+extern "C" int jllm_concat_rows(const float* a, const float* b, int n_rows, int d, void* out, int out_dtype, int ldo,
+                                hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (d <= 0 || ldo < 2 * d) JLLM_FAIL("concat_rows: rows of %d into rows of %d", d, ldo);
+  JLLM_DISPATCH_1(out_dtype, TO, { concat_rows_kernel<TO><<<n_rows, 256, 0, stream>>>(a, b, d, (TO*)out, ldo); })
+  JLLM_CHECK_LAUNCH("concat_rows");
+  return 0;
+}

@@ -3,7 +3,7 @@
 // fp32. A request's rows of a step are consecutive and in order (row_req ascends), so every kernel finds a request's
 // rows in the step by itself and the same launches serve portions of prompts, single rows and steps of fixed size.
 //
-//   short_conv_silu      y[t, c] = silu(sum_j taps[c, K - 1 - j] x[t - j, c]); inputs before the step's first row of a
+//   short_conv_silu      y[t, c] = silu(sum_j taps[c, K - 1 - j] x[t - j, c] (+ bias[c])); inputs before the step's first row of a
 //                        request come from that request's state, inputs before position 0 are the state's zeros
 //   short_conv_advance   the state's K - 1 inputs per channel move on by the request's rows of this step
 //   delta_prepare        per (row, key head), what the recurrence would otherwise compute in every lane of every wave:
@@ -33,7 +33,7 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void short_conv_silu_kernel(const T* __restrict__ x, int ldx, T* __restrict__ y, int ldy,
                                                               int channels, int taps, const TW* __restrict__ w,
-                                                              const float* __restrict__ state,
+                                                              const TW* __restrict__ bias, const float* __restrict__ state,
                                                               const int* __restrict__ row_req,
                                                               const int* __restrict__ state_slots) {
   const int t = blockIdx.x;
@@ -44,6 +44,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const T* __restric
   while (m < taps - 1 && t - m - 1 >= 0 && row_req[t - m - 1] == req) ++m;
   const float* st = state + (size_t)state_slots[req] * (taps - 1) * channels;
   float acc = 0.f;
+  const float shift = bias ? ldf(bias, c) : 0.f;
   for (int j = taps - 1; j >= 0; --j) {  // oldest input first
     float v;
     if (j <= m)
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const T* __restric
       v = st[(size_t)(taps - 1 - (j - m)) * channels + c];
     acc = fmaf(ldf(w, (size_t)c * taps + (taps - 1 - j)), v, acc);
   }
-  stf(y + (size_t)t * ldy, c, silu_f(acc));
+  stf(y + (size_t)t * ldy, c, silu_f(acc + shift));
 }
 
 // first row and number of rows of request `req` in the ascending list row_req[0 .. n)
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(256) void short_conv_advance_kernel(const T* __rest
 }
 
 extern "C" int jllm_short_conv(const void* x, int ldx, void* y, int ldy, int dtype, int n_rows, int n_requests, int channels,
-                               int taps, const void* w, int w_dtype, float* state, const int* row_req,
+                               int taps, const void* w, const void* bias, int w_dtype, float* state, const int* row_req,
                                const int* state_slots, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) JLLM_FAIL("short_conv: %d channels, %d taps (1..%d taps are taken)", channels, taps, CONV_MAX_TAPS);
@@ -106,7 +107,7 @@ extern "C" int jllm_short_conv(const void* x, int ldx, void* y, int ldy, int dty
   JLLM_DISPATCH_1(dtype, T, {
     JLLM_DISPATCH_1(w_dtype, TW, {
       short_conv_silu_kernel<T, TW><<<dim3(n_rows, cb), 256, 0, stream>>>((const T*)x, ldx, (T*)y, ldy, channels, taps, (const TW*)w,
-                                                                          state, row_req, state_slots);
+                                                                          (const TW*)bias, state, row_req, state_slots);
     })
     if (taps > 1)
       short_conv_advance_kernel<T><<<dim3(n_requests, cb), 256, 0, stream>>>((const T*)x, ldx, channels, taps, state, row_req,
@@ -118,12 +119,15 @@ extern "C" int jllm_short_conv(const void* x, int ldx, void* y, int ldy, int dty
 
 // ---------------------------------------------------------------------------------------------------------------------
 
-// prep row: qn (kv_heads x dk) | kn (kv_heads x dk) | g (heads) | beta (heads) | q . k (kv_heads)
+// prep row: qn (kv_heads x dk) | kn (kv_heads x dk) | g (heads) | beta (heads) | q . k (kv_heads) | g per key channel
+// (heads x dk, only with `decay_rows`: the decay's input per head and key channel, fp32 [rows, ldd], with dt_bias of
+// heads x dk entries; the one number per head is then not written)
 template <typename T, typename TW>
 __global__ __launch_bounds__(64) void delta_prepare_kernel(const T* __restrict__ conv, int ldc, const T* __restrict__ proj,
                                                            int ldp, int a_off, int b_off, const TW* __restrict__ a_log,
                                                            const TW* __restrict__ dt_bias, float* __restrict__ prep, int ldq,
-                                                           int heads, int kv_heads, int dk) {
+                                                           int heads, int kv_heads, int dk,
+                                                           const float* __restrict__ decay_rows, int ldd) {
   const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
   const T* q = conv + (size_t)row * ldc + (size_t)g * dk;
   const T* k = conv + (size_t)row * ldc + (size_t)(kv_heads + g) * dk;
@@ -145,12 +149,26 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(const T* __restrict__
   float* tail = out + (size_t)2 * kv_heads * dk;
   for (int j = lane; j < per; j += 64) {
     const int h = g * per + j;
-    const float z = ldf(proj + (size_t)row * ldp, a_off + h) + ldf(dt_bias, h);
-    const float sp = z > 20.f ? z : log1pf(expf(z));
-    tail[h] = expf(-expf(ldf(a_log, h)) * sp);
+    if (!decay_rows) {
+      const float z = ldf(proj + (size_t)row * ldp, a_off + h) + ldf(dt_bias, h);
+      const float sp = z > 20.f ? z : log1pf(expf(z));
+      tail[h] = expf(-expf(ldf(a_log, h)) * sp);
+    }
     tail[heads + h] = 1.0f / (1.0f + expf(-ldf(proj + (size_t)row * ldp, b_off + h)));
   }
   if (lane == 0) tail[2 * heads + g] = qk * rq * rk;
+  if (decay_rows) {
+    float* gv = tail + 2 * heads + kv_heads;
+    for (int j = 0; j < per; ++j) {
+      const int h = g * per + j;
+      const float rate = expf(ldf(a_log, h));
+      for (int i = lane; i < dk; i += 64) {
+        const float z = decay_rows[(size_t)row * ldd + (size_t)h * dk + i] + ldf(dt_bias, (size_t)h * dk + i);
+        const float sp = z > 20.f ? z : log1pf(expf(z));
+        gv[(size_t)h * dk + i] = expf(-rate * sp);
+      }
+    }
+  }
 }
 
 struct GdrArgs {
@@ -175,12 +193,15 @@ __device__ __forceinline__ float row16_sum(float d) {  // over a row of 16 lanes
 }
 
 // thread = wave * 64 + c * 16 + part: column blockIdx.z * 16 + wave * 4 + c, key rows part * E .. + E
-template <typename T, int E>
+// CHANNEL: the decay is a vector over the key channels (S's rows) instead of one number per head:
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q = (diag(g) S_old)^T q + (k . q) u
+template <typename T, int E, bool CHANNEL>
 __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   constexpr int C = GDR_CHUNK;
   constexpr int DKP = GDR_PARTS * E;              // the key size, padded with zeros
-  constexpr int ROWF = 2 * DKP + GDR_COLS + 4;    // q | k | v of the workgroup's columns | g | beta | q . k | -
-  constexpr int NQK = C * 2 * DKP / 256;
+  constexpr int NV = CHANNEL ? 3 : 2;             // vectors over the key size per row: q | k (| g)
+  constexpr int ROWF = NV * DKP + GDR_COLS + 4;   // q | k (| g) | v of the workgroup's columns | g | beta | q . k | -
+  constexpr int NQK = C * NV * DKP / 256;
   __shared__ __align__(16) float sm[C * ROWF];
   const int tid = threadIdx.x;
   const int part = tid & 15, cw = tid >> 4;  // cw: the column within the workgroup
@@ -201,6 +222,7 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   const T* conv = (const T*)A.conv;
   const size_t q_at = (size_t)kvh * dk, k_at = (size_t)(A.kv_heads + kvh) * dk;
   const size_t tail_at = (size_t)2 * A.kv_heads * dk;
+  const size_t g_at = tail_at + 2 * A.heads + A.kv_heads + (size_t)h * dk;
   const size_t v_at = (size_t)2 * A.kv_heads * dk + (size_t)h * A.dv + col0;
   float rqk[NQK], rv, rs;
   auto request = [&](int r0) {  // rows r0 .. r0 + C of the request, as far as it has them
@@ -208,9 +230,9 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
 #pragma unroll
     for (int j = 0; j < NQK; ++j) {
       const int idx = tid + 256 * j;
-      const int t = idx / (2 * DKP), w = idx % (2 * DKP);
+      const int t = idx / (NV * DKP), w = idx % (NV * DKP);
       const int i = w % DKP;
-      rqk[j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + (w < DKP ? q_at : k_at) + i] : 0.f;
+      rqk[j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + (w < DKP ? q_at : w < 2 * DKP ? k_at : g_at) + i] : 0.f;
     }
     {
       const int t = tid / GDR_COLS, cc = tid % GDR_COLS;
@@ -226,10 +248,10 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
 #pragma unroll
     for (int j = 0; j < NQK; ++j) {
       const int idx = tid + 256 * j;
-      sm[(idx / (2 * DKP)) * ROWF + idx % (2 * DKP)] = rqk[j];
+      sm[(idx / (NV * DKP)) * ROWF + idx % (NV * DKP)] = rqk[j];
     }
-    sm[(tid / GDR_COLS) * ROWF + 2 * DKP + tid % GDR_COLS] = rv;
-    if (tid < 3 * C) sm[(tid / 3) * ROWF + 2 * DKP + GDR_COLS + tid % 3] = rs;
+    sm[(tid / GDR_COLS) * ROWF + NV * DKP + tid % GDR_COLS] = rv;
+    if (tid < 3 * C) sm[(tid / 3) * ROWF + NV * DKP + GDR_COLS + tid % 3] = rs;
   };
   request(0);
   for (int r0 = 0; r0 < n; r0 += C) {
@@ -246,19 +268,33 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
         q[e] = row[i0 + e];
         k[e] = row[DKP + i0 + e];
       }
-      const float v = row[2 * DKP + cw], g = row[2 * DKP + GDR_COLS], beta = row[2 * DKP + GDR_COLS + 1];
-      const float qk = row[2 * DKP + GDR_COLS + 2];
-      float sk_ = 0.f, sq_ = 0.f;
+      const float v = row[NV * DKP + cw], g = row[NV * DKP + GDR_COLS], beta = row[NV * DKP + GDR_COLS + 1];
+      const float qk = row[NV * DKP + GDR_COLS + 2];
+      float sk_ = 0.f, sq_ = 0.f, o;
+      if constexpr (CHANNEL) {
 #pragma unroll
-      for (int e = 0; e < E; ++e) {
-        sk_ = fmaf(S[e], k[e], sk_);
-        sq_ = fmaf(S[e], q[e], sq_);
+        for (int e = 0; e < E; ++e) {
+          S[e] *= row[2 * DKP + i0 + e];
+          sk_ = fmaf(S[e], k[e], sk_);
+          sq_ = fmaf(S[e], q[e], sq_);
+        }
+        sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
+        const float u = beta * (v - sk_);
+        o = fmaf(qk, u, sq_);
+#pragma unroll
+        for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, S[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          sk_ = fmaf(S[e], k[e], sk_);
+          sq_ = fmaf(S[e], q[e], sq_);
+        }
+        sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
+        const float u = beta * (v - g * sk_);
+        o = fmaf(g, sq_, qk * u);
+#pragma unroll
+        for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, g * S[e]);
       }
-      sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
-      const float u = beta * (v - g * sk_);
-      const float o = fmaf(g, sq_, qk * u);
-#pragma unroll
-      for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, g * S[e]);
       if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = o;
     }
   }
@@ -267,29 +303,40 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
     if (col_on && i0 + e < dk) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
 }
 
-// prep: fp32 scratch [rows, >= 2 kv_heads dk + 2 heads + kv_heads]
+// prep: fp32 scratch [rows, >= 2 kv_heads dk + 2 heads + kv_heads (+ heads dk with decay_rows)]. decay_rows: null (one
+// decay per head, from proj at a_off, dt_bias of heads entries) or fp32 [rows, ldd] with the decay's input per head and
+// key channel (dt_bias of heads x dk entries)
 extern "C" int jllm_gated_delta(const void* qkv, int ldc, const void* proj, int ldp, int a_off, int b_off, int dtype,
                                 const void* a_log, const void* dt_bias, int w_dtype, float* prep, int ldq, float* state,
                                 float* out, int ldo, const int* row_req, const int* state_slots, int n_rows, int n_requests,
-                                int heads, int kv_heads, int dk, int dv, hipStream_t stream) {
+                                int heads, int kv_heads, int dk, int dv, const float* decay_rows, int ldd,
+                                hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 65535) JLLM_FAIL("gated_delta: %d heads over %d key heads", heads, kv_heads);
   if (dk <= 0 || dk > GDR_PARTS * 16 || dv <= 0 || dv > GDR_COLS * 65535) JLLM_FAIL("gated_delta: key size %d (1..%d are taken), value size %d", dk, GDR_PARTS * 16, dv);
   if (n_requests <= 0 || n_requests > n_rows) JLLM_FAIL("gated_delta: %d requests in %d rows", n_requests, n_rows);
-  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || ldp < a_off + heads || ldp < b_off + heads || a_off < 0 || b_off < 0 ||
-      ldq < 2 * kv_heads * dk + 2 * heads + kv_heads)
+  const bool channel = decay_rows != nullptr;
+  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || (!channel && (ldp < a_off + heads || a_off < 0)) ||
+      ldp < b_off + heads || b_off < 0 || ldq < 2 * kv_heads * dk + 2 * heads + kv_heads + (channel ? heads * dk : 0) ||
+      (channel && ldd < heads * dk))
     JLLM_FAIL("gated_delta: short rows");
   JLLM_DISPATCH_1(dtype, T, {
     JLLM_DISPATCH_1(w_dtype, TW, {
       delta_prepare_kernel<T, TW><<<dim3(n_rows, kv_heads), 64, 0, stream>>>((const T*)qkv, ldc, (const T*)proj, ldp, a_off, b_off,
                                                                             (const TW*)a_log, (const TW*)dt_bias, prep, ldq, heads,
-                                                                            kv_heads, dk);
+                                                                            kv_heads, dk, decay_rows, ldd);
     })
   })
   GdrArgs A{qkv, ldc, prep, ldq, state, out, ldo, row_req, state_slots, n_rows, heads, kv_heads, dk, dv};
   dim3 grid(n_requests, heads, (dv + GDR_COLS - 1) / GDR_COLS);
   const int per_lane = (dk + GDR_PARTS - 1) / GDR_PARTS;
-#define GDR_LAUNCH(E) gated_delta_kernel<T, E><<<grid, 256, 0, stream>>>(A)
+#define GDR_LAUNCH(E)                                                    \
+  do {                                                                   \
+    if (channel)                                                         \
+      gated_delta_kernel<T, E, true><<<grid, 256, 0, stream>>>(A);       \
+    else                                                                 \
+      gated_delta_kernel<T, E, false><<<grid, 256, 0, stream>>>(A);      \
+  } while (0)
   JLLM_DISPATCH_1(dtype, T, {
     if (per_lane <= 2)
       GDR_LAUNCH(2);

@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   __shared__ float red[4];
   const int t = blockIdx.x;
   const T* row = y + (size_t)t * ldy;
-  {
+  if (q_rank > 0) {  // a mixer without a query latent has nothing to norm here
     float ss = 0.f;
     for (int i = threadIdx.x; i < q_rank; i += 256) {
       const float v = ldf(row, q_off + i);
@@ -74,7 +74,8 @@ extern "C" int jllm_latent_prepare(const void* y, int dtype, int ldy, int n_rows
                                    float eps, const int* positions, const int* slots, const float* cos_t,
                                    const float* sin_t, void* cq, int ldcq, void* cache, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (q_rank <= 0 || ldcq < q_rank || q_off < 0 || q_off + q_rank > ldy) JLLM_FAIL("latent_prepare: query latent of %d at %d in rows of %d", q_rank, q_off, ldy);
+  if (q_rank == 0 && !cache) return 0;
+  if (q_rank < 0 || (q_rank > 0 && !cq) || ldcq < q_rank || q_off < 0 || q_off + q_rank > ldy) JLLM_FAIL("latent_prepare: query latent of %d at %d in rows of %d", q_rank, q_off, ldy);
   if (cache) {
     if (R <= 0 || Dr < 0 || kv_off < 0 || kv_off + R + Dr > ldy) JLLM_FAIL("latent_prepare: latent of %d + %d at %d in rows of %d", R, Dr, kv_off, ldy);
     if (rot_dims < 0 || rot_dims > Dr || (rot_dims & 1)) JLLM_FAIL("latent_prepare: %d rotated dims of %d", rot_dims, Dr);

@@ -1,6 +1,12 @@
-// A mixture of experts whose routing is a table: row t's experts are table[token[t]][0 .. top). Everything happens
-// on the device, from the token ids, so a step needs no answer from the GPU before it launches (and can be captured).
+// A mixture of experts whose routing is a table: row t's experts are table[token[t]][0 .. top) (a table by token id),
+// or table[t][0 .. top) where a router chose them for this step's rows (`tokens` null). Everything happens on the
+// device, so a step needs no answer from the GPU before it launches (and can be captured).
 //
+//   moe_router    one wave per row, from the router's fp32 logits z [T, E]: s = sigmoid(z); choice = s + correction;
+//                 the experts form `groups` equal groups of neighbours, a group's score is the sum of its two largest
+//                 choice scores and only the `keep` best groups can be chosen from; the `top` largest choice scores
+//                 among those win (the lowest index among equals); weights = s of the chosen / (their sum + 1e-20) *
+//                 scale. Writes the chosen experts [T, top] (int32) and their weights [T, top] (fp32)
 //   moe_route     one workgroup: counts the assignments (row, k) of every expert, lays them out expert by expert in
 //                 `sorted`, and cuts each expert's run into tiles of at most `tile_rows` rows: tiles[i] = (expert,
 //                 first place in `sorted`, rows); the tiles no expert needs have 0 rows
@@ -9,7 +15,8 @@
 //                 function to the two sums and writes hidden rows in the order of `sorted`; the second reads those
 //                 and writes fp32 rows by assignment, or, with top = 1, adds them straight into the residual rows
 //   moe_combine   residual[t] += weight * sum_k y[t * top + k], k ascending (or y[place_of[t * top + k]] where the second
-//                 product wrote its rows in the order of `sorted`)
+//                 product wrote its rows in the order of `sorted`); with `weights` [T, top] every term has its own
+//                 factor weights[t, k] as well
 //
 // The order of `sorted` within an expert comes from LDS atomics and may differ between runs; no result depends on it
 // (every output is one accumulator over ascending k of its own row and weight row). This file is the fp32 path
@@ -36,7 +43,7 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int*
   }
   __syncthreads();
   for (int a = threadIdx.x; a < A; a += MOE_ROUTE_THREADS) {
-    const int e = table[(size_t)tokens[a / top] * top + a % top];
+    const int e = table[(size_t)(tokens ? tokens[a / top] : a / top) * top + a % top];
     atomicAdd(&count[e], 1);
   }
   __syncthreads();
@@ -53,7 +60,7 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int*
   }
   __syncthreads();
   for (int a = threadIdx.x; a < A; a += MOE_ROUTE_THREADS) {
-    const int e = table[(size_t)tokens[a / top] * top + a % top];
+    const int e = table[(size_t)(tokens ? tokens[a / top] : a / top) * top + a % top];
     const int place = start[e] + atomicAdd(&cursor[e], 1);
     sorted[place] = a;
     if (place_of) place_of[a] = place;
@@ -188,23 +195,108 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
 
 // ---------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
-                                                         int top, float weight, const int* __restrict__ place_of) {
+                                                         int top, float weight, const int* __restrict__ place_of,
+                                                         const float* __restrict__ weights) {
   const int t = blockIdx.x;
   for (int i = threadIdx.x; i < width; i += 256) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) {
       const size_t row = place_of ? (size_t)place_of[t * top + k] : (size_t)t * top + k;
-      s += y[row * width + i];
+      s = weights ? fmaf(weights[(size_t)t * top + k], y[row * width + i], s) : s + y[row * width + i];
     }
     residual[(size_t)t * width + i] += weight * s;
   }
 }
 
 extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, const int* place_of,
-                                hipStream_t stream) {
+                                const float* weights, hipStream_t stream) {
   if (T <= 0) return 0;
   if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights);
   JLLM_CHECK_LAUNCH("moe_combine");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// LDS: s [E] | choice [E] | group score [groups] | group allowed [groups]
+template <typename TC>
+__global__ __launch_bounds__(64) void moe_router_kernel(const float* __restrict__ z, int ldz, const TC* __restrict__ correction,
+                                                       int E, int groups, int keep, int top, float scale,
+                                                       int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float rs[];
+  float* s = rs;
+  float* choice = rs + E;
+  float* gscore = rs + 2 * E;
+  int* allowed = (int*)(rs + 2 * E + groups);
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int per = E / groups;
+  for (int e = lane; e < E; e += 64) {
+    const float v = 1.0f / (1.0f + expf(-z[(size_t)t * ldz + e]));
+    s[e] = v;
+    choice[e] = v + (correction ? ldf(correction, e) : 0.f);
+  }
+  __syncthreads();
+  for (int g = lane; g < groups; g += 64) {  // the sum of the group's two largest choice scores
+    float a = -INFINITY, b = -INFINITY;
+    for (int i = 0; i < per; ++i) {
+      const float v = choice[g * per + i];
+      if (v > a) b = a, a = v; else if (v > b) b = v;
+    }
+    gscore[g] = per > 1 ? a + b : a;
+    allowed[g] = 0;
+  }
+  __syncthreads();
+  if (lane == 0) {
+    for (int n = 0; n < keep; ++n) {
+      int best = -1;
+      for (int g = 0; g < groups; ++g)
+        if (!allowed[g] && (best < 0 || gscore[g] > gscore[best])) best = g;
+      if (best >= 0) allowed[best] = 1;
+    }
+  }
+  __syncthreads();
+  for (int e = lane; e < E; e += 64)
+    if (!allowed[e / per]) choice[e] = -INFINITY;
+  __syncthreads();
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {  // ascending e: the lowest index among equals stays
+      const float v = choice[e];
+      if (v > bv) bv = v, bi = e;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+    }
+    if (bi >= E) bi = 0;  // nothing left to choose from: the entry point refuses the configurations where this could be
+    const float sv = s[bi];
+    sum += sv;
+    if (lane == 0) {
+      chosen[(size_t)t * top + k] = bi;
+      weights[(size_t)t * top + k] = sv;  // the raw score; scaled below once the sum is known
+      choice[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = weights[(size_t)t * top + k] / (sum + 1e-20f) * scale;
+}
+
+extern "C" int jllm_moe_router(const float* z, int ldz, const void* correction, int c_dtype, int T, int E, int groups, int keep,
+                               int top, float scale, int* chosen, float* weights, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (E <= 0 || top <= 0 || top > E || ldz < E) JLLM_FAIL("moe_router: top %d of %d experts in rows of %d", top, E, ldz);
+  if (groups <= 0 || E % groups || keep <= 0 || keep > groups || keep * (E / groups) < top)
+    JLLM_FAIL("moe_router: %d experts in %d groups of which %d are kept, for top %d", E, groups, keep, top);
+  const size_t smem = (size_t)(2 * E + 2 * groups) * sizeof(float);
+  if (smem > 64 * 1024) JLLM_FAIL("moe_router: %d experts are more than this kernel's LDS holds", E);
+  JLLM_DISPATCH_1(c_dtype, TC, {
+    moe_router_kernel<TC><<<T, 64, smem, stream>>>(z, ldz, (const TC*)correction, E, groups, keep, top, scale, chosen, weights);
+  })
+  JLLM_CHECK_LAUNCH("moe_router");
   return 0;
 }

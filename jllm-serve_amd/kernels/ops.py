@@ -73,15 +73,19 @@ def _declare(lib) -> None:
         "jllm_latent_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
         "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
         "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
-        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P],
+        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P, _P],
+        "jllm_moe_router": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+        "jllm_concat_rows": [_P, _P, _I, _I, _P, _I, _I, _P],
+        "jllm_ssm_scan": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_gated_group_norm": [_P, _I, _P, _I, _I, _P, _I, _F, _I, _I, _I, _P, _I, _I, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
         "jllm_layernorm_seam": [_P, _P, _I, _I, _P, _I, _P, _I, _I, _F, _F, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _P],
         "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
         "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
         "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
         "jllm_heads_finish_split": [_P, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
-        "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
-        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P],
+        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -216,6 +220,20 @@ def embed(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.T
     _i32(ids, n, "token ids")
     out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
     _call("jllm_embed", _ptr(table), _code(table.dtype), _ptr(ids), _ptr(out), n, table.shape[1], float(scale), _stream())
+    return out
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[a | b] row by row in ``out_dtype``: two fp32 row sets of one shape side by side, as the input of one product."""
+    _dev(a, b)
+    for t in (a, b):
+        if t.dtype != torch.float32 or t.dim() != 2 or not t.is_contiguous():
+            raise KernelError("concat_rows takes contiguous fp32 [rows, width] tensors")
+    if a.shape != b.shape:
+        raise KernelError(f"concat_rows: {tuple(a.shape)} beside {tuple(b.shape)}")
+    n, d = a.shape
+    out = activation_rows(n, 2 * d, out_dtype, a.device)
+    _call("jllm_concat_rows", _ptr(a), _ptr(b), n, d, _ptr(out), _code(out_dtype), out.stride(0), _stream())
     return out
 
 
@@ -858,20 +876,25 @@ def latent_prepare(y: torch.Tensor, q_rank: int, gq: torch.Tensor, eps: float, *
     _dev(y, gq, gkv, positions, slots, cos, sin, cache)
     _rows2d(y, "latent projections")
     T = y.shape[0]
-    if gq.numel() != q_rank or not gq.is_contiguous():
-        raise KernelError(f"the query latent's gain has {gq.numel()} entries for {q_rank}")
-    cq = torch.empty((T, q_rank), dtype=y.dtype, device=y.device)
+    if q_rank == 0:  # no query latent: only the cached row is prepared
+        if cache is None:
+            raise KernelError("latent_prepare: neither a query latent nor a cache to store into")
+        cq = None
+    else:
+        if gq is None or gq.numel() != q_rank or not gq.is_contiguous():
+            raise KernelError(f"the query latent's gain has {0 if gq is None else gq.numel()} entries for {q_rank}")
+        cq = torch.empty((T, q_rank), dtype=y.dtype, device=y.device)
     if cache is not None:
         if cache.dtype != y.dtype or not cache.is_contiguous() or cache.dim() != 3 or cache.shape[2] != kv_rank + rot_dim:
             raise KernelError("the latent cache must be a contiguous [pages, page_size, kv_rank + rot_dim] tensor of the activations' type")
-        if gkv is None or gkv.numel() != kv_rank or not gkv.is_contiguous() or gkv.dtype != gq.dtype:
+        if gkv is None or gkv.numel() != kv_rank or not gkv.is_contiguous() or (gq is not None and gkv.dtype != gq.dtype):
             raise KernelError(f"the latent's gain must have {kv_rank} entries of the query gain's type")
         _i32(positions, T, "positions")
         _i32(slots, T, "slots")
         _tables(cos, sin, rot_dims)
     _call("jllm_latent_prepare", _ptr(y), _code(y.dtype), y.stride(0), T, 0, q_rank, kv_off, kv_rank, rot_dim, rot_dims,
-          _ptr(gq), _ptr(gkv), _code(gq.dtype), float(eps), _ptr(positions), _ptr(slots), _ptr(cos), _ptr(sin), _ptr(cq),
-          cq.stride(0), _ptr(cache), _stream())
+          _ptr(gq), _ptr(gkv), _code((gq if gq is not None else gkv).dtype), float(eps), _ptr(positions), _ptr(slots),
+          _ptr(cos), _ptr(sin), _ptr(cq), cq.stride(0) if cq is not None else 0, _ptr(cache), _stream())
     return cq
 
 
@@ -1267,17 +1290,20 @@ def check_gated_delta_shape(heads: int, kv_heads: int, dk: int, dv: int, taps: i
 
 
 def short_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor,
-               n_requests: int) -> torch.Tensor:
+               n_requests: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu of a causal convolution over time per channel on the first C columns of ``x`` [T, >= C] (a view with any
-    row stride), ``taps`` [C, K] with the last column for the current row. A request's rows are consecutive and in
+    row stride), ``taps`` [C, K] with the last column for the current row, plus ``bias`` [C] (of the taps' type) where
+    given. A request's rows are consecutive and in
     order; the inputs in front of its first row of this step come from ``state`` [slots, K - 1, C] (fp32, oldest
     first) at the request's slot, and the state then moves on by the step's rows. Returns [T, C]."""
-    _dev(x, taps, state, row_req, state_slots)
+    _dev(x, taps, state, row_req, state_slots, bias)
     _rows2d(x, "convolution input")
     T = x.shape[0]
     if taps.dim() != 2 or not taps.is_contiguous():
         raise KernelError("convolution taps must be a contiguous [channels, taps] tensor")
     C, K = taps.shape
+    if bias is not None and (bias.numel() != C or bias.dtype != taps.dtype or not bias.is_contiguous()):
+        raise KernelError(f"the convolution's bias must have {C} entries of the taps' type")
     if x.shape[1] < C:
         raise KernelError(f"convolution input rows have {x.shape[1]} entries for {C} channels")
     if state.dtype != torch.float32 or not state.is_contiguous() or (K > 1 and (state.dim() != 3 or state.shape[1:] != (K - 1, C))):
@@ -1288,19 +1314,22 @@ def short_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req
     if T == 0:
         return y
     _call("jllm_short_conv", _ptr(x), x.stride(0), _ptr(y), y.stride(0), _code(x.dtype), T, int(n_requests), C, K, _ptr(taps),
-          _code(taps.dtype), _ptr(state), _ptr(row_req), _ptr(state_slots), _stream())
+          _ptr(bias), _code(taps.dtype), _ptr(state), _ptr(row_req), _ptr(state_slots), _stream())
     return y
 
 
 def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
                 state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor, n_requests: int, heads: int,
-                kv_heads: int, dk: int, dv: int) -> torch.Tensor:
+                kv_heads: int, dk: int, dv: int, decay_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The gated delta rule over the step's rows, request by request and token by token, from and into ``state``
     [slots, heads, dk, dv] (fp32). ``qkv`` [T, kv_heads x dk | kv_heads x dk | heads x dv] are the convolved q, k, v;
     ``proj`` rows hold, at the given offsets, the inputs a and b of decay and write strength (heads each). Per head:
     q and k become unit vectors (q also / sqrt(dk)); beta = sigmoid(b); g = exp(-exp(a_log) softplus(a + dt_bias));
-    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Returns the raw o, fp32 [T, heads x dv]."""
-    _dev(qkv, proj, a_log, dt_bias, state, row_req, state_slots)
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Returns the raw o, fp32 [T, heads x dv]. With
+    ``decay_rows`` (fp32 [T, heads x dk]) the decay is one number per head and key channel, g = exp(-exp(a_log[h])
+    softplus(decay_rows + dt_bias)) with ``dt_bias`` of heads x dk entries, acting on the rows of S; ``a_off`` is unused."""
+    _dev(qkv, proj, a_log, dt_bias, state, row_req, state_slots, decay_rows)
+    channel = decay_rows is not None
     _rows2d(qkv, "convolved q, k, v")
     _rows2d(proj, "projection rows")
     T = qkv.shape[0]
@@ -1308,10 +1337,15 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a
         raise KernelError("the projection rows and the convolved rows must agree in rows and type")
     if qkv.shape[1] != 2 * kv_heads * dk + heads * dv:
         raise KernelError(f"convolved rows have {qkv.shape[1]} entries, expected {2 * kv_heads * dk + heads * dv}")
-    if max(a_off + heads, b_off + heads) > proj.shape[1] or min(a_off, b_off) < 0:
+    if channel:
+        _rows2d(decay_rows, "decay rows")
+        if decay_rows.dtype != torch.float32 or decay_rows.shape != (T, heads * dk):
+            raise KernelError(f"the decay rows must be fp32 {(T, heads * dk)}, got {tuple(decay_rows.shape)} {decay_rows.dtype}")
+        a_off = 0
+    if max(a_off + (0 if channel else heads), b_off + heads) > proj.shape[1] or min(a_off, b_off) < 0:
         raise KernelError("a or b lie outside the projection rows")
-    if a_log.numel() != heads or dt_bias.numel() != heads:
-        raise KernelError(f"a_log and dt_bias must have {heads} entries")
+    if a_log.numel() != heads or dt_bias.numel() != (heads * dk if channel else heads):
+        raise KernelError(f"a_log must have {heads} entries, dt_bias {heads * dk if channel else heads}")
     wd = _same_type("a_log and dt_bias", a_log, dt_bias)
     if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dk, dv):
         raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dk}, {dv}] tensor")
@@ -1321,10 +1355,81 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a
     if T == 0:
         return out
     # what the preparing kernel leaves for the recurrence: unit q and k, decay, write strength and q . k, in fp32
-    prep = torch.empty((T, 2 * kv_heads * dk + 2 * heads + kv_heads), dtype=torch.float32, device=qkv.device)
+    prep = torch.empty((T, 2 * kv_heads * dk + 2 * heads + kv_heads + (heads * dk if channel else 0)), dtype=torch.float32,
+                       device=qkv.device)
     _call("jllm_gated_delta", _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(a_off), int(b_off), _code(qkv.dtype),
           _ptr(a_log), _ptr(dt_bias), wd, _ptr(prep), prep.stride(0), _ptr(state), _ptr(out), out.stride(0), _ptr(row_req),
-          _ptr(state_slots), T, int(n_requests), heads, kv_heads, dk, dv, _stream())
+          _ptr(state_slots), T, int(n_requests), heads, kv_heads, dk, dv, _ptr(decay_rows),
+          decay_rows.stride(0) if channel else 0, _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ state-space recurrence
+
+MAX_SSM_STATE = 256    # state rows per head that the recurrence keeps in registers (csrc/ssm_scan.hip)
+
+
+def check_ssm_shape(heads: int, groups: int, state: int, dv: int, taps: int) -> None:
+    """Raises when the state-space kernels do not take these sizes (asked when a model is built)."""
+    if heads <= 0 or groups <= 0 or heads % groups != 0:
+        raise KernelError(f"state-space recurrence: {heads} heads over {groups} groups")
+    if not 1 <= taps <= MAX_CONV_TAPS:
+        raise KernelError(f"state-space recurrence: a convolution of {taps} taps (1..{MAX_CONV_TAPS} are taken)")
+    if not 0 < state <= MAX_SSM_STATE or dv <= 0:
+        raise KernelError(f"state-space recurrence: state size {state} (1..{MAX_SSM_STATE} are taken), value size {dv}")
+
+
+def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, a_log: torch.Tensor, dt_bias: torch.Tensor, skip: torch.Tensor,
+             state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor, n_requests: int, heads: int, groups: int,
+             n: int, dv: int) -> torch.Tensor:
+    """A selective state-space recurrence over the step's rows, request by request and token by token, from and into
+    ``state`` [slots, heads, n, dv] (fp32). ``xbc`` [T, heads x dv | groups x n | groups x n] are the convolved x, B, C;
+    ``proj`` rows hold the step sizes' input (heads entries) from ``dt_off`` on. Per head (its group's B and C):
+    dt = softplus(dt_in + dt_bias); S <- exp(-exp(a_log) dt) S + dt B x^T; y = S^T C + skip x. Returns y, fp32
+    [T, heads x dv]."""
+    _dev(xbc, proj, a_log, dt_bias, skip, state, row_req, state_slots)
+    _rows2d(xbc, "convolved x, B, C")
+    _rows2d(proj, "projection rows")
+    T = xbc.shape[0]
+    if proj.shape[0] != T or proj.dtype != xbc.dtype:
+        raise KernelError("the projection rows and the convolved rows must agree in rows and type")
+    if xbc.shape[1] != heads * dv + 2 * groups * n:
+        raise KernelError(f"convolved rows have {xbc.shape[1]} entries, expected {heads * dv + 2 * groups * n}")
+    if dt_off < 0 or dt_off + heads > proj.shape[1]:
+        raise KernelError("the step sizes lie outside the projection rows")
+    if a_log.numel() != heads or dt_bias.numel() != heads or skip.numel() != heads:
+        raise KernelError(f"a_log, dt_bias and the skip weights must have {heads} entries")
+    wd = _same_type("a_log, dt_bias and the skip weights", a_log, dt_bias, skip)
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, n, dv):
+        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {n}, {dv}] tensor")
+    _i32(row_req, T, "row -> request map")
+    _i32(state_slots, n_requests, "state slots")
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=xbc.device)
+    if T == 0:
+        return out
+    _call("jllm_ssm_scan", _ptr(xbc), xbc.stride(0), _ptr(proj), proj.stride(0), int(dt_off), _code(xbc.dtype), _ptr(a_log),
+          _ptr(dt_bias), _ptr(skip), wd, _ptr(state), _ptr(out), out.stride(0), _ptr(row_req), _ptr(state_slots), T,
+          int(n_requests), heads, groups, n, dv, _stream())
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """rmsnorm(y * silu(z)) * weight with the root mean square taken over each of ``groups`` equal parts of a row: ``y``
+    fp32 [T, width], ``z`` [T, width] (a view with any row stride), ``weight`` [width]. The gate comes before the norm."""
+    _dev(y, z, weight)
+    _rows2d(y, "rows to norm")
+    _rows2d(z, "gate rows")
+    T, width = y.shape
+    if y.dtype != torch.float32 or z.shape != (T, width):
+        raise KernelError(f"gated_group_norm: fp32 rows {tuple(y.shape)} with a gate of {tuple(z.shape)}")
+    if weight.numel() != width or not weight.is_contiguous() or groups <= 0 or width % groups:
+        raise KernelError(f"gated_group_norm: a weight of {weight.numel()} for rows of {width} in {groups} groups")
+    out = activation_rows(T, width, out_dtype, y.device)
+    if T == 0:
+        return out
+    _call("jllm_gated_group_norm", _ptr(y), y.stride(0), _ptr(z), z.stride(0), _code(z.dtype), _ptr(weight), _code(weight.dtype),
+          float(eps), T, width, int(groups), _ptr(out), _code(out_dtype), out.stride(0), _stream())
     return out
 
 
@@ -1346,12 +1451,34 @@ class MoeRouting:
         return self.tile_rows == MOE_TILE_ROWS_MANY
 
 
-def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int, many_ok: bool = False) -> MoeRouting:
-    """Groups the assignments (row t, k-th expert of its token) by expert, on the device. ``many_ok``: the caller's
+def moe_router(z: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float):
+    """From the router's fp32 logits ``z`` [T, experts]: s = sigmoid(z); the choice scores are s + ``correction``; the
+    experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest choice scores and
+    only the ``keep`` best groups can be chosen from; the ``top`` largest choice scores among those win. Returns the
+    chosen experts (int32 [T, top]) and their weights (fp32 [T, top]): s of the chosen / (their sum + 1e-20) * scale."""
+    _dev(z, correction)
+    _rows2d(z, "router logits")
+    if z.dtype != torch.float32:
+        raise KernelError("the router's logits are fp32")
+    T, E = z.shape
+    if correction is not None and (correction.numel() != E or not correction.is_contiguous()):
+        raise KernelError(f"the router's correction has {correction.numel()} entries for {E} experts")
+    chosen = torch.empty((T, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=z.device)
+    if T == 0:
+        return chosen, weights
+    _call("jllm_moe_router", _ptr(z), z.stride(0), _ptr(correction), _code(correction.dtype) if correction is not None else F32,
+          T, E, int(groups), int(keep), int(top), float(scale), _ptr(chosen), _ptr(weights), _stream())
+    return chosen, weights
+
+
+def moe_route(token_ids: Optional[torch.Tensor], table: torch.Tensor, experts: int, many_ok: bool = False) -> MoeRouting:
+    """Groups the assignments (row t, k-th expert of its token) by expert, on the device. ``token_ids`` None: row t's
+    experts are ``table[t]`` (what a router chose for this step's rows). ``many_ok``: the caller's
     products can go through the tiled matrix-core kernel (bf16, K a multiple of 64): steps that give the experts 64 rows
     or more each on average are then cut into tiles of 128 rows, all others into tiles of 16."""
     _dev(token_ids, table)
-    T = token_ids.numel()
+    T = token_ids.numel() if token_ids is not None else table.shape[0]
     _i32(token_ids, T, "token ids")
     if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
         raise KernelError("the routing table must be a contiguous int32 [vocab, top] tensor")
@@ -1404,16 +1531,19 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, w2: Optio
     return out
 
 
-def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float, place_of: Optional[torch.Tensor] = None) -> None:
+def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float, place_of: Optional[torch.Tensor] = None,
+                weights: Optional[torch.Tensor] = None) -> None:
     """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending); with ``place_of`` the k-th row of t is
-    y[place_of[t * top + k]]."""
-    _dev(y, residual, place_of)
+    y[place_of[t * top + k]]; with ``weights`` (fp32 [T, top]) the k-th term is also multiplied by weights[t, k]."""
+    _dev(y, residual, place_of, weights)
     T, width = residual.shape
     if y.dtype != torch.float32 or residual.dtype != torch.float32 or not y.is_contiguous() or not residual.is_contiguous() \
             or y.shape != (T * top, width):
         raise KernelError("moe_combine takes contiguous fp32 [T * top, width] rows and the fp32 residual [T, width]")
     _i32(place_of, T * top, "places")
-    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _stream())
+    if weights is not None and (weights.dtype != torch.float32 or not weights.is_contiguous() or weights.numel() != T * top):
+        raise KernelError("moe_combine: the weights must be a contiguous fp32 [T, top] tensor")
+    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _ptr(weights), _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -176,3 +176,44 @@ class SandwichBlock(Part):
 
 
 register_part("arrangement", "sandwich", SandwichBlock, replace=True)
+
+
+class ParallelBlock(Part):
+    """One norm, two readers: with h = norm_in(x), x += mixer(h) + ffn(h). Both sublayers add their output into the
+    fp32 stream themselves (the mixer first, then the feed-forward), so the sum is taken in the stream."""
+
+    chains_norms = False
+
+    def __init__(self, spec, prefix, build, positions):
+        ending = getattr(spec, "name_ending", ".weight")
+        self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}{ending}", build)
+        mixer_prefix = f"{prefix}.{spec.mixer_prefix}" if getattr(spec, "mixer_prefix", "") else prefix
+        self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, mixer_prefix, build, positions)
+        self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build) if spec.ffn is not None else None
+        self.parts = tuple(p for p in (self.norm_in, self.mixer, self.ffn) if p is not None)
+        self.capturable = all(getattr(p, "capturable", True) for p in self.parts)
+
+    def weight_specs(self):
+        return [w for p in self.parts for w in p.weight_specs()]
+
+    def load(self, get):
+        for p in self.parts:
+            p.load(get)
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def state_spec(self):
+        return self.mixer.state_spec()
+
+    def step_planners(self):
+        return [pl for p in self.parts for pl in (p.step_planners() if hasattr(p, "step_planners") else [])]
+
+    def forward(self, x, step, slot):
+        h = self.norm_in.forward(x)  # a tensor: both readers need the same rows
+        self.mixer.forward(h, x, step, slot)
+        if self.ffn is not None:
+            self.ffn.forward(h, x, step)
+
+
+register_part("arrangement", "parallel", ParallelBlock, replace=True)

@@ -12,7 +12,9 @@ A step is
      (``ops.gated_delta``; its value columns are spread over workgroups, so its read-out comes back raw),
   4. the heads' norm, gain and silu gate (``ops.heads_finish``, the kernel that ends attention heads too),
   5. the output product.
-The same launches serve portions of prompts and single rows: the recurrence visits a request's rows one after the
+With one decay per head and key channel (``spec.decay == "channel"``) the decay's input is a product of its own behind
+the stacked one (through a narrow middle, W_up (W_down h), whose first half rides in the stack), in fp32; the gate's
+input may pass such a middle too. The same launches serve portions of prompts and single rows: the recurrence visits a request's rows one after the
 other either way, so its result does not depend on how a prompt was cut.
 """
 from __future__ import annotations
@@ -35,13 +37,29 @@ class GatedDelta(Part):
             ops.check_gated_delta_shape(spec.heads, spec.kv_heads, spec.dim, spec.vdim, spec.conv)
         except ops.KernelError as e:
             raise ValueError(f"{prefix}: {e}") from None
+        if spec.decay not in ("head", "channel"):
+            raise ValueError(f"{prefix}: a decay per '{spec.decay}' is not built ('head' and 'channel' are)")
+        if spec.decay == "channel" and spec.decay_rank == 0:
+            raise ValueError(f"{prefix}: a decay per key channel takes its input through a narrow middle (decay_rank)")
+        if spec.gate_fn not in ops.HEAD_GATES:
+            raise ValueError(f"{prefix}: gate function '{spec.gate_fn}' ({sorted(ops.HEAD_GATES)} are built)")
         self.qk_dim = spec.kv_heads * spec.dim
         self.v_dim = spec.heads * spec.vdim
         self.channels = 2 * self.qk_dim + self.v_dim  # what passes the convolutions: q | k | v
+        self.decay_dim = spec.heads * spec.dim if spec.decay == "channel" else spec.heads
         self.gate_at = self.channels
-        self.a_at = self.gate_at + self.v_dim
-        self.b_at = self.a_at + spec.heads
-        self.w_in = self.taps = self.a_log = self.dt_bias = self.gain = self.w_o = None
+        # the stacked product's columns behind q | k | v: gate (or its middle) | decay (or its middle) | b; a middle
+        # whose size the checkpoint chooses (-1) is known once the weights are loaded
+        self.gate_cols = self.a_at = self.a_cols = self.b_at = None
+        if spec.gate_rank >= 0 and spec.decay_rank >= 0:
+            self._offsets(spec.gate_rank, spec.decay_rank)
+        self.w_in = self.taps = self.a_log = self.dt_bias = self.gain = self.w_o = self.w_gate_up = self.w_decay_up = None
+
+    def _offsets(self, gate_rank: int, decay_rank: int) -> None:
+        self.gate_cols = gate_rank if gate_rank else self.v_dim
+        self.a_at = self.gate_at + self.gate_cols
+        self.a_cols = decay_rank if decay_rank else self.decay_dim
+        self.b_at = self.a_at + self.a_cols
 
     def _name(self, which: str, suffix: str = "") -> str:
         return f"{self.prefix}.{getattr(self.spec.names, which)}{suffix}"
@@ -51,15 +69,32 @@ class GatedDelta(Part):
         sizes = (("q", self.qk_dim), ("k", self.qk_dim), ("v", self.v_dim))
         out = [WeightSpec(self._name(n), (w, d)) for n, w in sizes]
         out += [WeightSpec(self._name(n, nm.conv_suffix), (w, s.conv)) for n, w in sizes]
-        out += [WeightSpec(self._name("beta"), (s.heads, d)), WeightSpec(self._name("decay"), (s.heads, d)),
-                WeightSpec(self._name("a_log"), (s.heads,), init="bias"), WeightSpec(self._name("dt_bias"), (s.heads,), init="bias"),
-                WeightSpec(self._name("norm"), (s.vdim,), init="gain"), WeightSpec(self._name("gate"), (self.v_dim, d)),
-                WeightSpec(self._name("o"), (d, self.v_dim))]
+        out.append(WeightSpec(self._name("beta"), (s.heads, d)))
+        if s.decay_rank:
+            out += [WeightSpec(self._name("decay_down"), (s.decay_rank, d)),
+                    WeightSpec(self._name("decay_up"), (self.decay_dim, s.decay_rank))]
+        else:
+            out.append(WeightSpec(self._name("decay"), (self.decay_dim, d)))
+        if s.gate_rank:
+            out += [WeightSpec(self._name("gate_down"), (s.gate_rank, d)), WeightSpec(self._name("gate_up"), (self.v_dim, s.gate_rank))]
+        else:
+            out.append(WeightSpec(self._name("gate"), (self.v_dim, d)))
+        out += [WeightSpec(self._name("a_log"), (s.heads,), init="bias"), WeightSpec(self._name("dt_bias"), (self.decay_dim,), init="bias"),
+                WeightSpec(self._name("norm"), (s.vdim,), init="gain"), WeightSpec(self._name("o"), (d, self.v_dim))]
         return out
 
     def load(self, get):
-        nm = self.spec.names
-        stack = [get(self._name(n)) for n in ("q", "k", "v", "gate", "decay", "beta")]
+        s, nm = self.spec, self.spec.names
+        gate_in = get(self._name("gate_down" if s.gate_rank else "gate"))
+        decay_in = get(self._name("decay_down" if s.decay_rank else "decay"))
+        self.w_gate_up = get(self._name("gate_up")) if s.gate_rank else None
+        self.w_decay_up = get(self._name("decay_up")) if s.decay_rank else None
+        for up, down, what in ((self.w_gate_up, gate_in, "gate"), (self.w_decay_up, decay_in, "decay")):
+            if up is not None and up.shape[1] != down.shape[0]:
+                raise ValueError(f"{self.prefix}: the two halves of the {what}'s input disagree about their middle: "
+                                 f"{down.shape[0]} and {up.shape[1]}")
+        self._offsets(gate_in.shape[0] if s.gate_rank else 0, decay_in.shape[0] if s.decay_rank else 0)
+        stack = [get(self._name(n)) for n in ("q", "k", "v")] + [gate_in, decay_in, get(self._name("beta"))]
         dt = stack[0].dtype if all(t.dtype == stack[0].dtype for t in stack) else torch.float32
         self.w_in = pad_rows(torch.cat([t.to(dt) for t in stack], dim=0).contiguous())
         del stack
@@ -98,10 +133,22 @@ class GatedDelta(Part):
         s = self.spec
         matrix, tail = slot.state
         qkv = ops.short_conv(y, self.taps, tail, step.row_req, step.state_slots, step.n_requests)
-        o = ops.gated_delta(qkv, y, self.a_at, self.b_at, self.a_log, self.dt_bias, matrix, step.row_req, step.state_slots,
-                            step.n_requests, s.heads, s.kv_heads, s.dim, s.vdim)
+        exact = self.build.exact
+        decay_rows = None
+        if s.decay == "channel":  # what enters the recurrence besides the projections is fp32: the decay's input too
+            decay_rows = ops.gemm(y[:, self.a_at:self.a_at + self.a_cols], self.w_decay_up, out_dtype=torch.float32, exact=exact)
+            a_at = 0
+        elif s.decay_rank:
+            raise NotImplementedError("a decay per head through a narrow middle")
+        else:
+            a_at = self.a_at
+        o = ops.gated_delta(qkv, y, a_at, self.b_at, self.a_log, self.dt_bias, matrix, step.row_req, step.state_slots,
+                            step.n_requests, s.heads, s.kv_heads, s.dim, s.vdim, decay_rows=decay_rows)
+        gate = y[:, self.gate_at:self.gate_at + self.gate_cols]
+        if s.gate_rank:
+            gate = ops.gemm(gate, self.w_gate_up, out_dtype=self.build.dtype, exact=exact)
         return ops.heads_finish(o, s.heads, 1, s.vdim, self.build.dtype, normed=True, eps=s.eps, gain=self.gain,
-                                gate=y[:, self.gate_at:self.gate_at + self.v_dim], gate_fn="silu", out=out, out_mul=out_mul)
+                                gate=gate, gate_fn=s.gate_fn, out=out, out_mul=out_mul)
 
     def output(self, xb, step, slot):
         return ops.gemm(self.heads_rows(xb, step, slot), self.w_o, out_dtype=torch.float32, exact=self.build.exact)

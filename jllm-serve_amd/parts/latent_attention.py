@@ -59,10 +59,15 @@ class LatentAttention(Part):
         self.prefix = prefix
         self.build = build
         self.position = positions[spec.position] if spec.position is not None else None
-        if getattr(self.position, "pairing", "half") != "half":
-            raise ValueError(f"{prefix}: this mixer's kernels rotate the pairs (i, i + rotary_dim / 2) only")
         rot = self.position.rotary() if self.position is not None else None
         self.rot_dims = rot[2] if rot is not None else 0
+        # The kernels rotate the pairs (i, i + rotary_dim / 2). A checkpoint whose pairs are neighbours (2i, 2i + 1)
+        # runs on the same kernels with the rows of its rotated projections reordered at load (evens first, then
+        # odds): a score is a dot product of a rotated query part and a rotated key part, and reordering both the same
+        # way changes no dot product. The angles of pair i are the same in both layouts.
+        self.reorder = None
+        if getattr(self.position, "pairing", "half") == "interleaved" and self.rot_dims:
+            self.reorder = list(range(0, self.rot_dims, 2)) + list(range(1, self.rot_dims, 2)) + list(range(self.rot_dims, spec.rot_dim))
         try:
             ops.check_latent_shape(spec.heads, spec.kv_rank, spec.rot_dim, self.rot_dims)
         except ops.KernelError as e:
@@ -78,8 +83,11 @@ class LatentAttention(Part):
 
     def weight_specs(self):
         s, d = self.spec, self.build.hidden
-        out = [WeightSpec(self._name("dq"), (s.q_rank, d)), WeightSpec(self._name("dq_norm"), (s.q_rank,), init="gain"),
-               WeightSpec(self._name("uq"), (s.heads * (s.dim + s.rot_dim), s.q_rank))]
+        if s.q_rank > 0:
+            out = [WeightSpec(self._name("dq"), (s.q_rank, d)), WeightSpec(self._name("dq_norm"), (s.q_rank,), init="gain"),
+                   WeightSpec(self._name("uq"), (s.heads * (s.dim + s.rot_dim), s.q_rank))]
+        else:  # the query comes straight from the input
+            out = [WeightSpec(self._name("q"), (s.heads * (s.dim + s.rot_dim), d))]
         if s.owns_cache:
             out += [WeightSpec(self._name("dkv"), (self.kv_width, d)),
                     WeightSpec(self._name("dkv_norm"), (s.kv_rank,), init="gain")]
@@ -94,19 +102,34 @@ class LatentAttention(Part):
 
     def load(self, get):
         s = self.spec
-        stack = [get(self._name("dq"))]
+
+        def reordered(w, first, per, count):
+            """Rows first + j * per + reorder[i] of w in place of first + j * per + i, for j < count."""
+            if self.reorder is None:
+                return w
+            w = w.clone()
+            idx = torch.tensor(self.reorder, device=w.device)
+            for j in range(count):
+                at = first + j * per
+                w[at:at + len(self.reorder)] = w[at + idx]
+            return w
+
+        q_name = "uq" if s.q_rank > 0 else "q"
+        w_q = reordered(get(self._name(q_name)), s.dim, s.dim + s.rot_dim, s.heads)
+        stack = [get(self._name("dq"))] if s.q_rank > 0 else [w_q]
         if s.owns_cache:
-            stack.append(get(self._name("dkv")))
+            stack.append(reordered(get(self._name("dkv")), s.kv_rank, 0, 1))
             self.g_kv = get(self._name("dkv_norm"))
         if s.out_gate:
             stack.append(get(self._name("gate")))
         dt = stack[0].dtype if all(t.dtype == stack[0].dtype for t in stack) else torch.float32
         self.w_in = torch.cat([t.to(dt) for t in stack], dim=0).contiguous()  # [dq | dkv | g] rows
         del stack
-        self.g_q = get(self._name("dq_norm"))
-        if self.g_kv is not None and self.g_kv.dtype != self.g_q.dtype:
+        self.g_q = get(self._name("dq_norm")) if s.q_rank > 0 else None
+        if self.g_kv is not None and self.g_q is not None and self.g_kv.dtype != self.g_q.dtype:
             self.g_q, self.g_kv = self.g_q.float(), self.g_kv.float()
-        self.w_uq = get(self._name("uq"))
+        self.w_uq = w_q if s.q_rank > 0 else None
+        self.q_width = s.heads * (s.dim + s.rot_dim)
         # W_uk[h] is [dim, kv_rank]; the query side needs its transpose as a weight [N = kv_rank, K = dim] per head
         self.w_ukt = get(self._name("uk")).view(s.heads, s.dim, s.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = get(self._name("uv")).view(s.heads, s.vdim, s.kv_rank).contiguous()
@@ -137,15 +160,16 @@ class LatentAttention(Part):
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdims = rot if rot is not None else (None, None, 0)
         y = ops.gemm(xb, self.w_in, out_dtype=self.build.dtype, exact=exact)
-        kv_off = s.q_rank
-        gate_off = s.q_rank + (self.kv_width if s.owns_cache else 0)
+        kv_off = s.q_rank if s.q_rank > 0 else self.q_width
+        gate_off = kv_off + (self.kv_width if s.owns_cache else 0)
+        cq = None
         if s.owns_cache and slot.writes:
             cq = ops.latent_prepare(y, s.q_rank, self.g_q, s.eps, kv_off=kv_off, kv_rank=s.kv_rank, rot_dim=s.rot_dim,
                                     rot_dims=rdims, gkv=self.g_kv, positions=step.positions, slots=g.slots, cos=cos,
                                     sin=sin, cache=cache)
-        else:
+        elif s.q_rank > 0:
             cq = ops.latent_prepare(y, s.q_rank, self.g_q, s.eps)
-        q = ops.gemm(cq, self.w_uq, out_dtype=self.build.dtype, exact=exact)
+        q = ops.gemm(cq, self.w_uq, out_dtype=self.build.dtype, exact=exact) if s.q_rank > 0 else y[:, :self.q_width]
         qa = ops.latent_heads(q, self.w_ukt, tail=s.rot_dim, rot_dims=rdims, positions=step.positions, cos=cos, sin=sin,
                               exact=exact)
         lat = ops.latent_attention(qa, cache, g.block_table, step.row_req, step.positions, s.heads, s.kv_rank, s.window,

@@ -44,6 +44,9 @@ class DecoderModel:
             if e.add_before is not None:
                 self.stream_vector_rows[e.add_before.name] = e.add_before.rows
         self.stream_vectors = {}
+        # matrices that mix the stream with the embedding output before a run (ScheduleEntry.mix_before), by tensor name
+        self.stream_mix_names = sorted({e.mix_before.name for e in config.schedule if e.mix_before is not None})
+        self.stream_mixes = {}
         self.watch = None  # a function (run, x) called with the stream after every run (tests, debugging)
         # a part that walks the step's requests on the host sets ``capturable = False``; then decode steps are
         # never recorded as graphs
@@ -57,6 +60,7 @@ class DecoderModel:
         for p in self.positions:  # a position encoding may have tensors of its own (a learned table)
             specs += p.weight_specs() if hasattr(p, "weight_specs") else []
         specs += [WeightSpec(name, (rows, c.hidden), init="bias") for name, rows in self.stream_vector_rows.items()]
+        specs += [WeightSpec(name, (c.hidden, 2 * c.hidden)) for name in self.stream_mix_names]
         for l in self.layers:
             specs += l.weight_specs()
         specs += self.final_norm.weight_specs()
@@ -75,9 +79,14 @@ class DecoderModel:
             if hasattr(p, "load"):
                 p.load(get)
         self.stream_vectors = {name: get(name) for name in self.stream_vector_rows}
+        self.stream_mixes = {name: get(name) for name in self.stream_mix_names}
         for l in self.layers:
             l.load(get)
         self.final_norm.load(get)
+        if self.config.logit_scale != 1.0:  # head (s * n) = s * (head n): the scale rides on the final norm's output
+            if not hasattr(self.final_norm, "scale_output"):
+                raise ValueError(f"a logit scale needs a final norm that can scale its output, '{self.config.final_norm.kind}' cannot")
+            self.final_norm.scale_output(self.config.logit_scale)
         self.lm_head = get(names.head) if names.head in set(source.names()) else self.embed
 
     # -------------------------------------------------------------------------------------------- cache plan
@@ -106,10 +115,18 @@ class DecoderModel:
             if hasattr(p, "embed_add"):
                 p.embed_add(x, step)
         schedule = self.config.schedule
+        x0 = x.clone() if self.stream_mix_names else None  # the embedding output, for the runs that mix it back in
         carry = None  # the next block's input norm, when the block before prepared it (parts/block.py)
         added = False  # this run's vector already joined the stream (the block before added it on its way out)
         for run, e in enumerate(schedule):
             layer = self.layers[e.layer]
+            if e.mix_before is not None:
+                # x <- W [x; x0] (+ the run's vector, as the product's bias): a new stream tensor
+                vec = self._stream_vector(e.add_before) if e.add_before is not None and not added else None
+                x = ops.gemm(ops.concat_rows(x, x0, self.build.dtype), self.stream_mixes[e.mix_before.name], bias=vec,
+                             out=torch.empty_like(x), exact=self.build.exact)
+                added = True
+                carry = None
             if e.add_before is not None and not added:
                 ops.layernorm_seam(x, 0.0, add_vec=self._stream_vector(e.add_before))
                 carry = None
@@ -121,13 +138,13 @@ class DecoderModel:
                 nxt_e = schedule[run + 1] if run + 1 < len(schedule) else None
                 nxt = self.layers[nxt_e.layer] if nxt_e is not None else None
                 next_norm = getattr(nxt, "norm_in", None) if getattr(nxt, "chains_norms", False) else None
-                if nxt_e is not None and nxt_e.add_before is not None and self.watch is None \
+                if nxt_e is not None and nxt_e.add_before is not None and nxt_e.mix_before is None and self.watch is None \
                         and getattr(layer, "takes_stream_vector", False):
                     carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm,
                                           add_after=self._stream_vector(nxt_e.add_before))
                     added = True
                 else:
-                    if nxt_e is not None and nxt_e.add_before is not None:
+                    if nxt_e is not None and (nxt_e.add_before is not None or nxt_e.mix_before is not None):
                         next_norm = None  # the stream changes before the next block reads it
                     carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm)
             if self.watch is not None:

@@ -13,7 +13,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.schema import TableMoeSpec
+from ..config.schema import RoutedMoeSpec, TableMoeSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import BuildContext, Part, part_factory, register_part
@@ -90,3 +90,75 @@ class TableMoe(Part):
 
 
 register_part("ffn", "table_moe", TableMoe, replace=True)
+
+
+class RoutedMoe(Part):
+    """A mixture of experts chosen by a router: x += sum over the row's chosen experts of weight * expert(xb).
+
+    The router's logits are an fp32 product of the rows with the router's weight (held in fp32); ``ops.moe_router`` turns
+    them into the chosen experts and their weights per row (sigmoid scores, a correction on the choice, groups of
+    experts of which only the best are open, weights normalised over the chosen). From there on the step is the
+    table-routed one with the step's own table: ``ops.moe_route`` groups the assignments by expert, the grouped products
+    run gate/up and down, ``ops.moe_combine`` takes the weighted sum into the residual. Nothing waits for the GPU, so a
+    decode step with this feed-forward can be captured."""
+
+    def __init__(self, spec: RoutedMoeSpec, prefix: str, build: BuildContext):
+        if not 0 < spec.top <= spec.experts or spec.experts % spec.groups or not 0 < spec.keep <= spec.groups \
+                or spec.top > spec.keep * (spec.experts // spec.groups):
+            raise ValueError(f"{prefix}: top {spec.top} of {spec.experts} experts in {spec.groups} groups, {spec.keep} kept")
+        if spec.activation not in ops.GATE_FUNCTIONS or spec.activation == "swish_clamped":
+            raise ValueError(f"{prefix}: gate function '{spec.activation}' is not one of this feed-forward's (silu, gelu_tanh)")
+        self.spec = spec
+        self.prefix = prefix
+        self.build = build
+        self.gate = ops.GATE_FUNCTIONS[spec.activation]
+        self.takes_normed_rows = False
+        self.w_gate = self.w_up = self.w_down = self.w_router = self.correction = None
+
+    def _expert(self, e: int, which: str) -> str:
+        n = self.spec.names
+        return f"{self.prefix}.{n.expert}{e}.{getattr(n, which)}{n.ending}"
+
+    def _own(self, which: str) -> str:
+        return f"{self.prefix}.{getattr(self.spec.names, which)}{self.spec.names.ending}"
+
+    def weight_specs(self):
+        s, d = self.spec, self.build.hidden
+        out = []
+        for e in range(s.experts):
+            out += [WeightSpec(self._expert(e, "gate"), (s.hidden, d)), WeightSpec(self._expert(e, "up"), (s.hidden, d)),
+                    WeightSpec(self._expert(e, "down"), (d, s.hidden))]
+        out.append(WeightSpec(self._own("router"), (s.experts, d)))
+        if s.correction:
+            out.append(WeightSpec(self._own("correction"), (s.experts,), init="bias"))
+        return out
+
+    def load(self, get):
+        s = self.spec
+        stack = lambda which: torch.stack([get(self._expert(e, which)) for e in range(s.experts)]).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        self.w_router = get(self._own("router")).float().contiguous()  # the routing is computed in fp32
+        self.correction = get(self._own("correction")).float().contiguous() if s.correction else None
+
+    def forward(self, xb, residual, step, then_norm=None):
+        s, exact = self.spec, self.build.exact
+        T = xb.shape[0]
+        z = ops.gemm(xb, self.w_router, out_dtype=torch.float32, exact=True)  # plain FMAs in fp32 in both run types
+        chosen, weights = ops.moe_router(z, self.correction, s.groups, s.keep, s.top, s.scale)
+        many_ok = not exact and self.build.dtype == torch.bfloat16 and self.w_gate.dtype == torch.bfloat16 \
+            and residual.shape[1] % 64 == 0 and s.hidden % 64 == 0
+        routing = ops.moe_route(None, chosen, s.experts, many_ok=many_ok)
+        A = T * s.top
+        hidden = torch.empty((A, s.hidden), dtype=self.build.dtype, device=xb.device)
+        ops.moe_gemm(xb, self.w_gate, routing, w2=self.w_up, out=hidden, in_map=1, out_map=0, gate=self.gate, exact=exact)
+        y = torch.empty((A, residual.shape[1]), dtype=torch.float32, device=xb.device)
+        if routing.many:
+            ops.moe_gemm(hidden, self.w_down, routing, out=y, in_map=0, out_map=0, exact=exact)
+            ops.moe_combine(y, residual, s.top, 1.0, place_of=routing.place_of, weights=weights)
+        else:
+            ops.moe_gemm(hidden, self.w_down, routing, out=y, in_map=0, out_map=1, exact=exact)
+            ops.moe_combine(y, residual, s.top, 1.0, weights=weights)
+        return None
+
+
+register_part("ffn", "routed_moe", RoutedMoe, replace=True)

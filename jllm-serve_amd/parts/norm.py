@@ -2,6 +2,8 @@
 weight and a bias: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b."""
 from __future__ import annotations
 
+import torch
+
 from ..config.schema import LayerNormSpec, NormSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
@@ -29,6 +31,11 @@ class RMSNorm(Part):
         """The normalised rows as a promise, for consumers that feed them to ``ops.gemm`` only."""
         return ops.NormedRows(x, self.gain, self.eps, self.out_dtype)
 
+    def scale_output(self, factor: float) -> None:
+        """From now on the norm's output is ``factor`` times what it was (the gain in fp32)."""
+        if factor != 1.0:
+            self.gain = (self.gain.float() * factor).contiguous()
+
     def after_add(self, a, w, residual, bias=None, exact=False):
         """residual += a @ w.T (+ bias), and this norm of the result as a promise: the product that makes the new
         residual rows can prepare their norm on its way out (``ops.gemm_add_then_norm``)."""
@@ -47,17 +54,30 @@ class LayerNorm(Part):
         self.eps = float(spec.eps)
         self.dim = dim
         self.weight_name = weight_name
+        self.has_bias = bool(getattr(spec, "bias", True))
         self.bias_name = weight_name + spec.bias_suffix
         self.out_dtype = build.dtype
         self.gain = self.bias = None
 
     def weight_specs(self):
-        return [WeightSpec(self.weight_name, (self.dim,), init="gain"), WeightSpec(self.bias_name, (self.dim,), init="bias")]
+        out = [WeightSpec(self.weight_name, (self.dim,), init="gain")]
+        if self.has_bias:
+            out.append(WeightSpec(self.bias_name, (self.dim,), init="bias"))
+        return out
 
     def load(self, get):
-        self.gain, self.bias = get(self.weight_name), get(self.bias_name)
+        self.gain = get(self.weight_name)
+        # a norm without a bias runs the same kernel with zeros in its place
+        self.bias = get(self.bias_name) if self.has_bias else torch.zeros_like(self.gain)
         if self.gain.dtype != self.bias.dtype:
             self.gain, self.bias = self.gain.float(), self.bias.float()
+
+    def scale_output(self, factor: float) -> None:
+        """From now on the norm's output is ``factor`` times what it was (weight and bias in fp32): for a product
+        behind it whose result is scaled by a constant."""
+        if factor != 1.0:
+            self.gain = (self.gain.float() * factor).contiguous()
+            self.bias = (self.bias.float() * factor).contiguous()
 
     def forward(self, x, rows=None):
         return ops.layernorm_seam(x, self.eps, nxt=(self.gain, self.bias), out_dtype=self.out_dtype, rows=rows)

@@ -41,12 +41,23 @@ class WeightError(ValueError):
 class WeightSpec:
     """One tensor a part needs. ``init`` tells the random-weights mode how to fill it:
     "matrix" N(0, std), "gain" 1 + N(0, gain_std), "bias" N(0, std), "zeros", "expert_table" (int32 [rows, top]:
-    every row holds ``top`` different expert numbers below the count that the tensor's name is registered with)."""
+    every row holds ``top`` different expert numbers below the count that the tensor's name is registered with). A
+    dimension of -1 is the checkpoint's to choose (a narrow middle between two projections whose size no config key
+    gives): any size matches, the part that declared it checks that its tensors agree, and the random-weights mode
+    takes ``free`` for it."""
 
     name: str
     shape: Tuple[int, ...]
     init: str = "matrix"
     optional: bool = False
+    free: int = 16
+
+    def matches(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(e == -1 or e == g for e, g in zip(self.shape, shape))
+
+    def concrete(self) -> Tuple[int, ...]:
+        return tuple(self.free if e == -1 else e for e in self.shape)
 
 
 def check(specs: Sequence[WeightSpec], source, where: str = "") -> None:
@@ -56,7 +67,7 @@ def check(specs: Sequence[WeightSpec], source, where: str = "") -> None:
     unexpected = sorted(have - wanted)
     wrong = []
     for s in specs:
-        if s.name in have and tuple(source.shape(s.name)) != tuple(s.shape):
+        if s.name in have and not s.matches(source.shape(s.name)):
             wrong.append((s.name, tuple(source.shape(s.name)), tuple(s.shape)))
     if missing or unexpected or wrong:
         raise WeightError(missing, unexpected, wrong, where)
@@ -127,13 +138,15 @@ class RandomSource:
         return list(self.specs)
 
     def shape(self, name: str) -> Tuple[int, ...]:
-        return self.specs[name].shape
+        return self.specs[name].concrete()
 
     def dtype(self, name: str) -> torch.dtype:
         return torch.int32 if self.specs[name].init == "expert_table" else self._dtype
 
     def get(self, name: str) -> torch.Tensor:
         s = self.specs[name]
+        if -1 in s.shape:
+            s = WeightSpec(s.name, s.concrete(), s.init, s.optional, s.free)
         g = torch.Generator(device=self.device)
         g.manual_seed((self.seed * 1000003 + zlib.crc32(name.encode("utf-8"))) % (2**63 - 1))
         if s.init == "zeros":
