@@ -184,6 +184,19 @@ def moe(h: torch.Tensor, mlp: dict, w: Dict[str, torch.Tensor]):
     return out
 
 
+def mixer(h: torch.Tensor, weights: Dict[str, torch.Tensor], i: int, layer: dict, eps: float, positions: torch.Tensor):
+    """Layer i's mixer alone on the input rows h of one sequence."""
+    mw = _sub(weights, f"l{i}.mix.")
+    kind = layer["type"]
+    if kind == "latent_attention":
+        return latent_attention(h, layer["mixer"], mw, eps, positions)
+    if kind == "channel_delta":
+        return channel_delta(h, layer["mixer"], mw, eps)
+    if kind == "mamba2":
+        return mamba2(h, layer["mixer"], mw, eps)
+    raise ValueError(kind)
+
+
 # ----------------------------------------------------------------------------------------------- the model
 
 
@@ -218,16 +231,7 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
             x = linear(torch.cat([x, x0], dim=-1), W["loop.in"]) + W["loop.step"][t]
         layer = cfg["layers"][i]
         h = layer_norm(x, W[f"l{i}.norm1"], eps)
-        mw = _sub(W, f"l{i}.mix.")
-        kind = layer["type"]
-        if kind == "latent_attention":
-            y = latent_attention(h, layer["mixer"], mw, eps, positions)
-        elif kind == "channel_delta":
-            y = channel_delta(h, layer["mixer"], mw, eps)
-        elif kind == "mamba2":
-            y = mamba2(h, layer["mixer"], mw, eps)
-        else:
-            raise ValueError(kind)
+        y = mixer(h, W, i, layer, eps, positions)
         if layer.get("mlp") is not None:
             y = y + moe(h, layer["mlp"], _sub(W, f"l{i}.mlp."))
         x = x + y
@@ -235,3 +239,12 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
             streams.append(x.clone())
     xn = layer_norm(x, W["final.norm"], eps)
     return linear(xn, W["head"]) * float(cfg.get("logit_scale", 1.0))
+
+
+def greedy(cfg: dict, weights: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
+    """The n_new tokens that follow the prompt when the largest logit (the lowest index among equals) is always taken."""
+    toks = list(prompt)
+    for _ in range(n_new):
+        row = forward(cfg, weights, toks)[-1]
+        toks.append(int(torch.argmax(row)))
+    return toks[len(prompt):]
