@@ -19,6 +19,9 @@ main decode run a sampled one.
 
 `--workload compare --design kebepel [--size 2k|4k]` measures a Kebepel model (parallel attention / delta-rule layers and
 differential attention layers) beside the Qwen3 dense model of the same width, heads and feed-forward.
+`--workload compare --design ratasun [--size 2k|4k]` measures a Ratasun model (latent attention, a delta rule with a decay
+per key channel and a state-space layer, every layer with router-chosen experts beside the mixer) beside the Miforax
+model of the same width, heads, latent and experts.
 `--workload compare [--size 2k|4k]` is another run altogether: a Miforax model (latent attention with a window, dense
 and table-routed expert layers in turn) beside the closest model the engine had before, a Qwen3 dense model with the
 same width, layers, heads, window and feed-forward width, both with random weights: prefill of 2,048 tokens and
@@ -224,6 +227,97 @@ class KebepelWork:
         return rows * (2.0 * self.per_row + self.row_flops) + self.pair_flops * pairs + 2.0 * self.V * self.d * selected
 
 
+RATASUN_EXTRA = {  # what a Ratasun model has beyond the sizes it shares with the Miforax model of the same name
+    "2k": dict(d_heads=16, d_kv_heads=8, d_dim=128, d_vdim=128, conv=4, middle=16, s_heads=64, s_vdim=64, s_state=128,
+               s_groups=8, s_norm_groups=8, groups=4, keep=2),
+    "4k": dict(d_heads=32, d_kv_heads=16, d_dim=128, d_vdim=128, conv=4, middle=16, s_heads=128, s_vdim=64, s_state=128,
+               s_groups=8, s_norm_groups=8, groups=8, keep=4),
+}
+
+
+def ratasun_config(z: dict) -> dict:
+    """Four layers: latent attention, delta rule, state-space layer, latent attention, every one with routed experts
+    (top x expert_ff weights per token) beside the mixer; no loop."""
+    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot"], "vdim": z["vdim"], "kv_rank": z["kv_rank"],
+              "scale": (z["dim"] + z["rot"]) ** -0.5, "rot": {"base": 1e6, "dims": z["rot"]}}
+    delta = {"heads": z["d_heads"], "kv_heads": z["d_kv_heads"], "dim": z["d_dim"], "vdim": z["d_vdim"], "conv": z["conv"]}
+    ssm = {"heads": z["s_heads"], "vdim": z["s_vdim"], "state": z["s_state"], "groups": z["s_groups"],
+           "norm_groups": z["s_norm_groups"], "conv": z["conv"]}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"], "scale": 2.5, "groups": {"count": z["groups"], "keep": z["keep"]}},
+           "expert": {"ff": z["expert_ff"]}}
+    kinds = [("latent_attention", latent), ("channel_delta", delta), ("mamba2", ssm), ("latent_attention", latent)]
+    return {"architecture": "Ratasun", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "max_positions": 8192, "layers": [{"type": k, "mixer": m, "mlp": moe} for k, m in kinds]}
+
+
+class RatasunWork:
+    """Bytes and flops of passes over a Ratasun model of the sizes ``z`` (the interface of ``Work``). A decode step
+    reads every weight outside the experts, of the experts at most batch x top per layer, per request the cached latent
+    rows of the attention layers, and reads and writes the matrices of the two recurrent layers (fp32); a row costs 2
+    flops per weight it passes through, per (row, key) pair and head 2 x (kv_rank + rot) for the score and 2 x kv_rank
+    for the weighted sum, and in the recurrences 6 x (key or state size) x value size per head."""
+
+    def __init__(self, z: dict, dtype: str):
+        self.z = z
+        self.L, self.d, self.H, self.Hkv, self.F, self.V = 4, z["width"], z["heads"], 1, z["top"] * z["expert_ff"], z["vocab"]
+        self.hd = z["kv_rank"] + z["rot"]
+        self.esize = 2 if dtype == "bf16" else 4
+        self.dtype = dtype
+        d, H, r = self.d, self.H, z["kv_rank"]
+        latent = (H * (z["dim"] + z["rot"]) + r + z["rot"]) * d + H * z["dim"] * r + H * z["vdim"] * r + d * H * z["vdim"]
+        dh, dg, dk, dv, mid = z["d_heads"], z["d_kv_heads"], z["d_dim"], z["d_vdim"], z["middle"]
+        delta = (2 * dg * dk + dh * dv + dh + 2 * mid) * d + mid * (dh * dk + dh * dv) + d * dh * dv
+        inner = z["s_heads"] * z["s_vdim"]
+        ssm = (2 * inner + 2 * z["s_groups"] * z["s_state"] + z["s_heads"]) * d + d * inner
+        self.mixers = 2 * latent + delta + ssm
+        self.expert = 3 * d * z["expert_ff"]
+        self.router = z["experts"] * d
+        self.kv_bytes_per_token = 2 * self.hd * self.esize
+        self.state_bytes = (dh * dk * dv + z["s_heads"] * z["s_state"] * z["s_vdim"]) * 4 * 2
+        self.row_flops = 6 * dh * dk * dv + 6 * z["s_heads"] * z["s_state"] * z["s_vdim"]
+        self.weight_bytes = (self.mixers + self.L * (self.router + z["experts"] * self.expert) + self.V * d) * self.esize
+
+    def decode_bytes(self, tokens_held: float, batch: int = 0) -> float:
+        z = self.z
+        touched = min(z["experts"], max(batch, 1) * z["top"])
+        w = self.mixers + self.L * (self.router + touched * self.expert) + self.V * self.d
+        return w * self.esize + self.kv_bytes_per_token * tokens_held + self.state_bytes * max(batch, 1)
+
+    def pairs(self, T: int) -> float:
+        return T * (T + 1) / 2.0
+
+    def flops(self, rows: float, pairs: float, selected: float) -> float:
+        per_row = self.mixers + self.L * (self.router + self.z["top"] * self.expert)
+        return rows * (2.0 * per_row + self.row_flops) + 2.0 * 2 * self.H * (self.hd + self.z["kv_rank"]) * pairs \
+            + 2.0 * self.V * self.d * selected
+
+
+def compare_ratasun(args) -> dict:
+    """``--workload compare --design ratasun``: the Ratasun model of ``--size`` and the Miforax model of the same width,
+    heads, latent and experts, one after the other: prefill of 2,048 tokens in one portion, decoding at batch 8 and 64
+    behind prompts of 1,152 tokens."""
+    z = {**COMPARE_SIZES[args.size], **RATASUN_EXTRA[args.size]}
+    ctx = 4096
+    decodes = [dict(key=f"b{B}", batch=B, prompt_len=1152, steps=args.point_steps, warmup=4) for B in (8, 64)]
+    prefills = [dict(key="main", tokens=2048, portion=2048)]
+    out = {"metric": f"Ratasun beside Miforax at equal sizes ({args.size})", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "higher_is_better": True,
+           "config": {"size": args.size, **z, "context": ctx, "page_size": PAGE}, "models": {}}
+    for name, shape, work in (("ratasun", ratasun_config(z), RatasunWork(z, "bf16")),
+                              ("miforax", miforax_config(z), LatentWork(z, "bf16"))):
+        r = steady(args, name, "bf16", 0, ctx, decodes, prefills, shape=shape, work=work)
+        m = {"prefill_2048_tok_s": r["prefill"]["main"]["value"], "prefill_2048_ms": r["prefill"]["main"]["ms"],
+             "prefill_flop_frac": r["prefill"]["main"]["frac"]}
+        for B in (8, 64):
+            s_, held, by = r["decode"][f"b{B}"]
+            m[f"decode_b{B}_tok_s"] = round(B / s_, 1)
+            m[f"decode_b{B}_ms"] = round(s_ * 1e3, 3)
+            m[f"decode_b{B}_hbm_frac"] = round(by / s_ / HBM_PEAK, 4)
+        out["models"][name] = m
+    out["value"] = out["models"]["ratasun"]["decode_b8_tok_s"]
+    return out
+
+
 def compare_kebepel(args) -> dict:
     """``--workload compare --design kebepel``: the Kebepel model of ``--size`` and the Qwen3 dense model of the same
     width, heads, head size and feed-forward, one after the other: prefill of 2,048 tokens in one portion, decoding at
@@ -398,8 +492,9 @@ def main() -> int:
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end; "
                          "compare: a Miforax model beside the Qwen3 dense model of the same sizes")
     ap.add_argument("--size", default="2k", choices=sorted(COMPARE_SIZES), help="compare: which sizes")
-    ap.add_argument("--design", default="miforax", choices=["miforax", "kebepel"],
-                    help="compare: which design stands beside the Qwen3 dense model of the same sizes")
+    ap.add_argument("--design", default="miforax", choices=["miforax", "kebepel", "ratasun"],
+                    help="compare: which design stands beside the Qwen3 dense model of the same sizes (ratasun: beside the "
+                         "Miforax model of the same sizes)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -409,7 +504,8 @@ def main() -> int:
         print(json.dumps(serve_workload(args)))
         return 0
     if args.workload == "compare":
-        print(json.dumps(compare_kebepel(args) if args.design == "kebepel" else compare_workload(args)))
+        run = {"kebepel": compare_kebepel, "ratasun": compare_ratasun}.get(args.design, compare_workload)
+        print(json.dumps(run(args)))
         return 0
 
     import torch

@@ -201,7 +201,8 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   constexpr int DKP = GDR_PARTS * E;              // the key size, padded with zeros
   constexpr int NV = CHANNEL ? 3 : 2;             // vectors over the key size per row: q | k (| g)
   constexpr int ROWF = NV * DKP + GDR_COLS + 4;   // q | k (| g) | v of the workgroup's columns | g | beta | q . k | -
-  constexpr int NQK = C * NV * DKP / 256;
+  constexpr int NJ = C * DKP / 256;               // entries of one vector of a chunk per thread
+  constexpr int NQK = NV * NJ;
   __shared__ __align__(16) float sm[C * ROWF];
   const int tid = threadIdx.x;
   const int part = tid & 15, cw = tid >> 4;  // cw: the column within the workgroup
@@ -228,11 +229,14 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   auto request = [&](int r0) {  // rows r0 .. r0 + C of the request, as far as it has them
     const int have = min(C, n - r0);
 #pragma unroll
-    for (int j = 0; j < NQK; ++j) {
-      const int idx = tid + 256 * j;
-      const int t = idx / (NV * DKP), w = idx % (NV * DKP);
-      const int i = w % DKP;
-      rqk[j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + (w < DKP ? q_at : w < 2 * DKP ? k_at : g_at) + i] : 0.f;
+    for (int v = 0; v < NV; ++v) {  // vector by vector, so that every index below is a shift and a mask
+      const size_t at = v == 0 ? q_at : v == 1 ? k_at : g_at;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int idx = tid + 256 * j;
+        const int t = idx / DKP, i = idx % DKP;
+        rqk[v * NJ + j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + at + i] : 0.f;
+      }
     }
     {
       const int t = tid / GDR_COLS, cc = tid % GDR_COLS;
@@ -246,9 +250,12 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   };
   auto stage = [&]() {
 #pragma unroll
-    for (int j = 0; j < NQK; ++j) {
-      const int idx = tid + 256 * j;
-      sm[(idx / (NV * DKP)) * ROWF + idx % (NV * DKP)] = rqk[j];
+    for (int v = 0; v < NV; ++v) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int idx = tid + 256 * j;
+        sm[(idx / DKP) * ROWF + v * DKP + idx % DKP] = rqk[v * NJ + j];
+      }
     }
     sm[(tid / GDR_COLS) * ROWF + NV * DKP + tid % GDR_COLS] = rv;
     if (tid < 3 * C) sm[(tid / 3) * ROWF + NV * DKP + GDR_COLS + tid % 3] = rs;

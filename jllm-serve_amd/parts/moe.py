@@ -16,7 +16,7 @@ import torch
 from ..config.schema import RoutedMoeSpec, TableMoeSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import BuildContext, Part, part_factory, register_part
+from .base import BuildContext, Part, pad_rows, part_factory, register_part
 
 
 class TableMoe(Part):
@@ -137,13 +137,19 @@ class RoutedMoe(Part):
         s = self.spec
         stack = lambda which: torch.stack([get(self._expert(e, which)) for e in range(s.experts)]).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
-        self.w_router = get(self._own("router")).float().contiguous()  # the routing is computed in fp32
+        # The routing is computed in fp32. A router stored in bf16 stays bf16 in a bf16 run: the product of two bf16
+        # numbers is exact in fp32 and the product kernels sum in fp32, so the logits are the fp32 ones (up to the
+        # order of the sums) and the product runs on the matrix cores; its rows are filled up to a group of 16.
+        w = get(self._own("router"))
+        fast = w.dtype == torch.bfloat16 and self.build.dtype == torch.bfloat16 and not self.build.exact
+        self.w_router = pad_rows(w) if fast else w.float().contiguous()
         self.correction = get(self._own("correction")).float().contiguous() if s.correction else None
 
     def forward(self, xb, residual, step, then_norm=None):
         s, exact = self.spec, self.build.exact
         T = xb.shape[0]
-        z = ops.gemm(xb, self.w_router, out_dtype=torch.float32, exact=True)  # plain FMAs in fp32 in both run types
+        # fp32 logits: plain FMAs for an fp32 router, the matrix cores' exact products for a bf16 one
+        z = ops.gemm(xb, self.w_router, out_dtype=torch.float32, exact=self.w_router.dtype == torch.float32)[:, :s.experts]
         chosen, weights = ops.moe_router(z, self.correction, s.groups, s.keep, s.top, s.scale)
         many_ok = not exact and self.build.dtype == torch.bfloat16 and self.w_gate.dtype == torch.bfloat16 \
             and residual.shape[1] % 64 == 0 and s.hidden % 64 == 0
