@@ -9,9 +9,10 @@
 //                     only needs x[j]), so a workgroup of four waves owns 16 value columns of one head of one request:
 //                     16 lanes per column with a sixteenth of the state rows each; sums over a column's lanes are moves
 //                     inside a row of 16 lanes. Rows are requested in chunks of 16 a chunk ahead and shared through
-//                     LDS; dt and the decay of a chunk's rows are computed once per chunk by 16 lanes. The walk over a
-//                     request's rows is one instruction sequence whatever the cut of the prompt, so fp32 results do
-//                     not depend on it.
+//                     LDS; dt and the decay of a chunk's rows are computed once per chunk by 16 lanes. A token's
+//                     arithmetic is one sequence of operations whatever the cut of the prompt (the tokens of a full
+//                     chunk are only interleaved, their sums over the lanes taken together), so fp32 results do not
+//                     depend on it.
 //   gated_group_norm  out = rmsnorm_g(y * silu(z)) * w: the gate comes first, then every one of `groups` equal parts
 //                     of a row is divided by its own root mean square
 #include <math.h>
@@ -128,18 +129,36 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
     __syncthreads();
     if (r0 + C < n) request(r0 + C);  // in flight while this chunk is worked through
     const int have = min(C, n - r0);
-    for (int t = 0; t < have; ++t) {
+    // one token: the lane's rows of S move on and give its part of the read-out. No lane needs another's numbers for
+    // the state (unlike the delta rule, whose write depends on a sum over the rows), so a full chunk's tokens are
+    // worked through without a wait between them and their sums over the lanes are taken together afterwards; a
+    // token's arithmetic is the same either way.
+    auto token = [&](int t) {
       const float* row = sm + t * ROWF;
-      const float x = row[2 * NP + cw], dt = row[2 * NP + SSM_COLS], dA = row[2 * NP + SSM_COLS + 1];
-      const float dx = dt * x;
+      const float dx = row[2 * NP + SSM_COLS] * row[2 * NP + cw], dA = row[2 * NP + SSM_COLS + 1];
       float y = 0.f;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         S[e] = fmaf(dx, row[i0 + e], dA * S[e]);
         y = fmaf(S[e], row[NP + i0 + e], y);
       }
-      y = ssm_row16_sum(y);
-      if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = fmaf(skip, x, y);
+      return y;
+    };
+    if (have == C) {
+      float yp[C];
+#pragma unroll
+      for (int t = 0; t < C; ++t) yp[t] = token(t);
+#pragma unroll
+      for (int t = 0; t < C; ++t) yp[t] = ssm_row16_sum(yp[t]);
+      float mine = yp[0];  // lane `part` of a column writes token `part`
+#pragma unroll
+      for (int t = 1; t < C; ++t) mine = part == t ? yp[t] : mine;
+      if (col_on) A.out[(size_t)(lo + r0 + part) * A.ldo + (size_t)h * A.dv + col] = fmaf(skip, sm[part * ROWF + 2 * NP + cw], mine);
+    } else {
+      for (int t = 0; t < have; ++t) {
+        const float y = ssm_row16_sum(token(t));
+        if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = fmaf(skip, sm[t * ROWF + 2 * NP + cw], y);
+      }
     }
   }
 #pragma unroll
