@@ -219,7 +219,13 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * dk * A.dv;
   float S[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) S[e] = (col_on && i0 + e < dk) ? S_at[(size_t)(i0 + e) * A.dv + col] : 0.f;
+  for (int e = 0; e < E; ++e) {
+    // every lane loads from a place that exists and drops what it does not own: a load inside a condition waits
+    // for the loads before it (its register is also written on the other path), and these would come one by one
+    const bool own = col_on && i0 + e < dk;
+    const float s = S_at[own ? (size_t)(i0 + e) * A.dv + col : 0];
+    S[e] = own ? s : 0.f;
+  }
   const T* conv = (const T*)A.conv;
   const size_t q_at = (size_t)kvh * dk, k_at = (size_t)(A.kv_heads + kvh) * dk;
   const size_t tail_at = (size_t)2 * A.kv_heads * dk;
@@ -235,17 +241,22 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
       for (int j = 0; j < NJ; ++j) {
         const int idx = tid + 256 * j;
         const int t = idx / DKP, i = idx % DKP;
-        rqk[v * NJ + j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + at + i] : 0.f;
+        const bool own = t < have && i < dk;
+        const float p = A.prep[(size_t)(lo + r0 + (own ? t : 0)) * A.ldq + at + (own ? i : 0)];
+        rqk[v * NJ + j] = own ? p : 0.f;
       }
     }
     {
       const int t = tid / GDR_COLS, cc = tid % GDR_COLS;
-      rv = (t < have && col0 + cc < A.dv) ? ldf(conv + (size_t)(lo + r0 + t) * A.ldc + v_at, cc) : 0.f;
+      const bool own = t < have && col0 + cc < A.dv;
+      const float p = ldf(conv + (size_t)(lo + r0 + (own ? t : 0)) * A.ldc + v_at, own ? cc : 0);
+      rv = own ? p : 0.f;
     }
-    rs = 0.f;
-    if (tid < 3 * C && tid / 3 < have) {
+    {
       const int which = tid % 3;  // g, beta, q . k
-      rs = A.prep[(size_t)(lo + r0 + tid / 3) * A.ldq + tail_at + (which == 0 ? h : which == 1 ? A.heads + h : 2 * A.heads + kvh)];
+      const bool own = tid < 3 * C && tid / 3 < have;
+      const float p = A.prep[(size_t)(lo + r0 + (own ? tid / 3 : 0)) * A.ldq + tail_at + (which == 0 ? h : which == 1 ? A.heads + h : 2 * A.heads + kvh)];
+      rs = own ? p : 0.f;
     }
   };
   auto stage = [&]() {

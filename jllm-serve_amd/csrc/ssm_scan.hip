@@ -85,7 +85,13 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
   float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * ns * A.dv;
   float S[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) S[e] = (col_on && i0 + e < ns) ? S_at[(size_t)(i0 + e) * A.dv + col] : 0.f;
+  for (int e = 0; e < E; ++e) {
+    // every lane loads from a place that exists and drops what it does not own: a load inside a condition waits
+    // for the loads before it (its register is also written on the other path), and these would come one by one
+    const bool own = col_on && i0 + e < ns;
+    const float s = S_at[own ? (size_t)(i0 + e) * A.dv + col : 0];
+    S[e] = own ? s : 0.f;
+  }
   const T* xbc = (const T*)A.xbc;
   const T* dtp = (const T*)A.dt;
   const size_t inner = (size_t)A.heads * A.dv;
@@ -100,13 +106,21 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
       const int idx = tid + 256 * j;
       const int t = idx / (2 * NP), w = idx % (2 * NP);
       const int i = w % NP;
-      rbc[j] = (t < have && i < ns) ? ldf(xbc + (size_t)(lo + r0 + t) * A.ld + (w < NP ? b_at : c_at), i) : 0.f;
+      const bool own = t < have && i < ns;
+      const float p = ldf(xbc + (size_t)(lo + r0 + (own ? t : 0)) * A.ld + (w < NP ? b_at : c_at), own ? i : 0);
+      rbc[j] = own ? p : 0.f;
     }
     {
       const int t = tid / SSM_COLS, cc = tid % SSM_COLS;
-      rx = (t < have && col0 + cc < A.dv) ? ldf(xbc + (size_t)(lo + r0 + t) * A.ld + x_at, cc) : 0.f;
+      const bool own = t < have && col0 + cc < A.dv;
+      const float p = ldf(xbc + (size_t)(lo + r0 + (own ? t : 0)) * A.ld + x_at, own ? cc : 0);
+      rx = own ? p : 0.f;
     }
-    rdt = (tid < C && tid < have) ? ldf(dtp + (size_t)(lo + r0 + tid) * A.ldt, A.dt_off + h) : 0.f;
+    {
+      const bool own = tid < C && tid < have;
+      const float p = ldf(dtp + (size_t)(lo + r0 + (own ? tid : 0)) * A.ldt, A.dt_off + h);
+      rdt = own ? p : 0.f;
+    }
   };
   auto stage = [&]() {
 #pragma unroll
