@@ -278,7 +278,11 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
     __syncthreads();
     if (r0 + C < n) request(r0 + C);  // in flight while this chunk is worked through
     const int have = min(C, n - r0);
-    for (int t = 0; t < have; ++t) {
+    // One token: the lane's rows of S move on; what it leaves are the lane's part of S^T q and (q . k) u. Only the sum
+    // behind u (S^T k over the lanes) stands between one token and the next, in two chains of multiply-adds; the
+    // read-out's sum over the lanes is taken afterwards, for a full chunk for all its tokens together. A token's
+    // arithmetic is the same sequence in a full chunk and in a short one.
+    auto token = [&](int t, float& sq_part, float& qu) {
       const float* row = sm + t * ROWF;
       float q[E], k[E];
 #pragma unroll
@@ -288,32 +292,53 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
       }
       const float v = row[NV * DKP + cw], g = row[NV * DKP + GDR_COLS], beta = row[NV * DKP + GDR_COLS + 1];
       const float qk = row[NV * DKP + GDR_COLS + 2];
-      float sk_ = 0.f, sq_ = 0.f, o;
+      float sk0 = 0.f, sk1 = 0.f, sq_ = 0.f;
       if constexpr (CHANNEL) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          S[e] *= row[2 * DKP + i0 + e];
-          sk_ = fmaf(S[e], k[e], sk_);
-          sq_ = fmaf(S[e], q[e], sq_);
-        }
-        sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
+        for (int e = 0; e < E; ++e) S[e] *= row[2 * DKP + i0 + e];
+      }
+#pragma unroll
+      for (int e = 0; e < E; e += 2) {
+        sk0 = fmaf(S[e], k[e], sk0);
+        sk1 = fmaf(S[e + 1], k[e + 1], sk1);
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) sq_ = fmaf(S[e], q[e], sq_);
+      const float sk_ = row16_sum(sk0 + sk1);
+      if constexpr (CHANNEL) {
         const float u = beta * (v - sk_);
-        o = fmaf(qk, u, sq_);
 #pragma unroll
         for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, S[e]);
+        qu = qk * u;
       } else {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          sk_ = fmaf(S[e], k[e], sk_);
-          sq_ = fmaf(S[e], q[e], sq_);
-        }
-        sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
         const float u = beta * (v - g * sk_);
-        o = fmaf(g, sq_, qk * u);
 #pragma unroll
         for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, g * S[e]);
+        qu = qk * u;
       }
-      if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = o;
+      sq_part = sq_;
+    };
+    auto read_out = [&](int t, float sq_sum, float qu) {  // o = S^T q after the token's write
+      if constexpr (CHANNEL) return sq_sum + qu;
+      return fmaf(sm[t * ROWF + NV * DKP + GDR_COLS], sq_sum, qu);
+    };
+    if (have == C) {
+      float sq[C], qu[C];
+#pragma unroll
+      for (int t = 0; t < C; ++t) token(t, sq[t], qu[t]);
+#pragma unroll
+      for (int t = 0; t < C; ++t) sq[t] = read_out(t, row16_sum(sq[t]), qu[t]);
+      float mine = sq[0];  // lane `part` of a column writes token `part`
+#pragma unroll
+      for (int t = 1; t < C; ++t) mine = part == t ? sq[t] : mine;
+      if (col_on) A.out[(size_t)(lo + r0 + part) * A.ldo + (size_t)h * A.dv + col] = mine;
+    } else {
+      for (int t = 0; t < have; ++t) {
+        float sq_part, qu;
+        token(t, sq_part, qu);
+        const float o = read_out(t, row16_sum(sq_part), qu);
+        if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = o;
+      }
     }
   }
 #pragma unroll
