@@ -58,6 +58,18 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const T* __restric
 
 // first row and number of rows of request `req` in the ascending list row_req[0 .. n)
 __device__ __forceinline__ void rows_of_request(const int* __restrict__ row_req, int n, int req, int& lo, int& cnt) {
+  if (req < n) {
+    // a step of single rows has request r's one row at place r: three loads side by side in place of two searches.
+    // In an ascending list, a place that holds r between two neighbours that do not is all of r's rows.
+    const int here = row_req[req];
+    const int before = req > 0 ? row_req[req - 1] : -1;
+    const int after = req + 1 < n ? row_req[req + 1] : 0x7fffffff;
+    if (here == req && before != req && after != req) {
+      lo = req;
+      cnt = 1;
+      return;
+    }
+  }
   int a = 0, b = n;
   while (a < b) {
     const int mid = (a + b) >> 1;
@@ -195,7 +207,10 @@ __device__ __forceinline__ float row16_sum(float d) {  // over a row of 16 lanes
 // thread = wave * 64 + c * 16 + part: column blockIdx.z * 16 + wave * 4 + c, key rows part * E .. + E
 // CHANNEL: the decay is a vector over the key channels (S's rows) instead of one number per head:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q = (diag(g) S_old)^T q + (k . q) u
-template <typename T, int E, bool CHANNEL>
+// FEW: the form for steps of few rows per request (decoding). It leaves out the interleaved walk over a full chunk, whose
+// registers would halve the workgroups that a compute unit holds: such a step is a wait for each request's state, and
+// the more workgroups wait at once, the more of it is in flight. A token's arithmetic is the same in both forms.
+template <typename T, int E, bool CHANNEL, bool FEW>
 __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   constexpr int C = GDR_CHUNK;
   constexpr int DKP = GDR_PARTS * E;              // the key size, padded with zeros
@@ -309,7 +324,7 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
         const float u = beta * (v - sk_);
 #pragma unroll
         for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, S[e]);
-        qu = qk * u;
+        qu = u;
       } else {
         const float u = beta * (v - g * sk_);
 #pragma unroll
@@ -319,10 +334,10 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
       sq_part = sq_;
     };
     auto read_out = [&](int t, float sq_sum, float qu) {  // o = S^T q after the token's write
-      if constexpr (CHANNEL) return sq_sum + qu;
+      if constexpr (CHANNEL) return fmaf(sm[t * ROWF + NV * DKP + GDR_COLS + 2], qu, sq_sum);  // (q . k) u + S^T q
       return fmaf(sm[t * ROWF + NV * DKP + GDR_COLS], sq_sum, qu);
     };
-    if (have == C) {
+    if (!FEW && have == C) {
       float sq[C], qu[C];
 #pragma unroll
       for (int t = 0; t < C; ++t) token(t, sq[t], qu[t]);
@@ -373,12 +388,17 @@ extern "C" int jllm_gated_delta(const void* qkv, int ldc, const void* proj, int 
   GdrArgs A{qkv, ldc, prep, ldq, state, out, ldo, row_req, state_slots, n_rows, heads, kv_heads, dk, dv};
   dim3 grid(n_requests, heads, (dv + GDR_COLS - 1) / GDR_COLS);
   const int per_lane = (dk + GDR_PARTS - 1) / GDR_PARTS;
-#define GDR_LAUNCH(E)                                                    \
-  do {                                                                   \
-    if (channel)                                                         \
-      gated_delta_kernel<T, E, true><<<grid, 256, 0, stream>>>(A);       \
-    else                                                                 \
-      gated_delta_kernel<T, E, false><<<grid, 256, 0, stream>>>(A);      \
+  const bool few = n_rows <= 2 * n_requests;
+#define GDR_LAUNCH(E)                                                           \
+  do {                                                                          \
+    if (channel && few)                                                         \
+      gated_delta_kernel<T, E, true, true><<<grid, 256, 0, stream>>>(A);        \
+    else if (channel)                                                           \
+      gated_delta_kernel<T, E, true, false><<<grid, 256, 0, stream>>>(A);       \
+    else if (few)                                                               \
+      gated_delta_kernel<T, E, false, true><<<grid, 256, 0, stream>>>(A);       \
+    else                                                                        \
+      gated_delta_kernel<T, E, false, false><<<grid, 256, 0, stream>>>(A);      \
   } while (0)
   JLLM_DISPATCH_1(dtype, T, {
     if (per_lane <= 2)

@@ -40,6 +40,18 @@ struct SsmArgs {
 };
 
 __device__ __forceinline__ void ssm_rows_of_request(const int* __restrict__ row_req, int n, int req, int& lo, int& cnt) {
+  if (req < n) {
+    // a step of single rows has request r's one row at place r: three loads side by side in place of two searches.
+    // In an ascending list, a place that holds r between two neighbours that do not is all of r's rows.
+    const int here = row_req[req];
+    const int before = req > 0 ? row_req[req - 1] : -1;
+    const int after = req + 1 < n ? row_req[req + 1] : 0x7fffffff;
+    if (here == req && before != req && after != req) {
+      lo = req;
+      cnt = 1;
+      return;
+    }
+  }
   int a = 0, b = n;
   while (a < b) {
     const int mid = (a + b) >> 1;
@@ -63,7 +75,10 @@ __device__ __forceinline__ float ssm_row16_sum(float d) {  // over a row of 16 l
 }
 
 // thread = cw * 16 + part: column blockIdx.z * 16 + cw, state rows part * E .. + E
-template <typename T, typename TW, int E>
+// FEW: the form for steps of few rows per request (decoding). It leaves out the interleaved walk over a full chunk, whose
+// registers would halve the workgroups that a compute unit holds: such a step is a wait for each request's state, and
+// the more workgroups wait at once, the more of it is in flight. A token's arithmetic is the same in both forms.
+template <typename T, typename TW, int E, bool FEW>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
   constexpr int C = SSM_CHUNK;
   constexpr int NP = SSM_PARTS * E;            // the state size, padded with zeros
@@ -158,7 +173,7 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
       }
       return y;
     };
-    if (have == C) {
+    if (!FEW && have == C) {
       float yp[C];
 #pragma unroll
       for (int t = 0; t < C; ++t) yp[t] = token(t);
@@ -192,7 +207,14 @@ extern "C" int jllm_ssm_scan(const void* xbc, int ld, const void* dt, int ldt, i
   SsmArgs A{xbc, ld, dt, ldt, dt_off, a_log, dt_bias, skip, state, out, ldo, row_req, state_slots, n_rows, heads, groups, n, dv};
   dim3 grid(n_requests, heads, (dv + SSM_COLS - 1) / SSM_COLS);
   const int per_lane = (n + SSM_PARTS - 1) / SSM_PARTS;
-#define SSM_LAUNCH(E) ssm_scan_kernel<T, TW, E><<<grid, 256, 0, stream>>>(A)
+  const bool few = n_rows <= 2 * n_requests;
+#define SSM_LAUNCH(E)                                              \
+  do {                                                             \
+    if (few)                                                       \
+      ssm_scan_kernel<T, TW, E, true><<<grid, 256, 0, stream>>>(A);  \
+    else                                                           \
+      ssm_scan_kernel<T, TW, E, false><<<grid, 256, 0, stream>>>(A); \
+  } while (0)
   JLLM_DISPATCH_1(dtype, T, {
     JLLM_DISPATCH_1(w_dtype, TW, {
       if (per_lane <= 2)
