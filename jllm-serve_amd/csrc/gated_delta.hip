@@ -188,7 +188,7 @@ struct GdrArgs {
   int ldc;
   const float* prep;  // [rows, ldq]: what delta_prepare left
   int ldq;
-  float* state;       // [slots, heads, dk, dv]
+  float* state;       // [slots, heads, dv, dk]: a head's matrix column by column
   float* out;         // [rows, ldo]: heads x dv, the raw read-out
   int ldo;
   const int* row_req;
@@ -233,13 +233,27 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
   const int i0 = part * E;
   float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * dk * A.dv;
   float S[E];
+  // A head's state lies column by column ([dv][dk]), so a lane's entries are side by side and a workgroup's 16 columns one
+  // run of memory. Every lane loads from a place that exists and drops what it does not own: a load inside a condition
+  // waits for the loads before it (its register is also written on the other path), and these would come one by one.
+  const bool wide = E >= 4 && (dk & 3) == 0;  // then a lane's entries start on 16 bytes and end with the column
+  if (wide) {
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    // every lane loads from a place that exists and drops what it does not own: a load inside a condition waits
-    // for the loads before it (its register is also written on the other path), and these would come one by one
-    const bool own = col_on && i0 + e < dk;
-    const float s = S_at[own ? (size_t)(i0 + e) * A.dv + col : 0];
-    S[e] = own ? s : 0.f;
+    for (int e = 0; e < E; e += 4) {
+      const bool own = col_on && i0 + e < dk;
+      const float4 s = *reinterpret_cast<const float4*>(S_at + (own ? (size_t)col * dk + i0 + e : 0));
+      S[e] = own ? s.x : 0.f;
+      S[(e + 1) % E] = own ? s.y : 0.f;
+      S[(e + 2) % E] = own ? s.z : 0.f;
+      S[(e + 3) % E] = own ? s.w : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool own = col_on && i0 + e < dk;
+      const float s = S_at[own ? (size_t)col * dk + i0 + e : 0];
+      S[e] = own ? s : 0.f;
+    }
   }
   const T* conv = (const T*)A.conv;
   const size_t q_at = (size_t)kvh * dk, k_at = (size_t)(A.kv_heads + kvh) * dk;
@@ -356,9 +370,16 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
       }
     }
   }
+  if (wide) {
 #pragma unroll
-  for (int e = 0; e < E; ++e)
-    if (col_on && i0 + e < dk) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
+    for (int e = 0; e < E; e += 4)
+      if (col_on && i0 + e < dk)
+        *reinterpret_cast<float4*>(S_at + (size_t)col * dk + i0 + e) = make_float4(S[e], S[(e + 1) % E], S[(e + 2) % E], S[(e + 3) % E]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (col_on && i0 + e < dk) S_at[(size_t)col * dk + i0 + e] = S[e];
+  }
 }
 
 // prep: fp32 scratch [rows, >= 2 kv_heads dk + 2 heads + kv_heads (+ heads dk with decay_rows)]. decay_rows: null (one

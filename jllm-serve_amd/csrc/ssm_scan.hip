@@ -31,7 +31,7 @@ struct SsmArgs {
   const void* a_log;  // [heads]
   const void* dt_bias;
   const void* skip;   // D [heads]
-  float* state;       // [slots, heads, n, dv]
+  float* state;       // [slots, heads, dv, n]: a head's matrix column by column
   float* out;         // [rows, ldo]: heads x dv
   int ldo;
   const int* row_req;
@@ -99,13 +99,27 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
   const int i0 = part * E;
   float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * ns * A.dv;
   float S[E];
+  // A head's state lies column by column ([dv][ns]), so a lane's entries are side by side and a workgroup's 16 columns one
+  // run of memory. Every lane loads from a place that exists and drops what it does not own: a load inside a condition
+  // waits for the loads before it (its register is also written on the other path), and these would come one by one.
+  const bool wide = E >= 4 && (ns & 3) == 0;  // then a lane's entries start on 16 bytes and end with the column
+  if (wide) {
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    // every lane loads from a place that exists and drops what it does not own: a load inside a condition waits
-    // for the loads before it (its register is also written on the other path), and these would come one by one
-    const bool own = col_on && i0 + e < ns;
-    const float s = S_at[own ? (size_t)(i0 + e) * A.dv + col : 0];
-    S[e] = own ? s : 0.f;
+    for (int e = 0; e < E; e += 4) {
+      const bool own = col_on && i0 + e < ns;
+      const float4 s = *reinterpret_cast<const float4*>(S_at + (own ? (size_t)col * ns + i0 + e : 0));
+      S[e] = own ? s.x : 0.f;
+      S[(e + 1) % E] = own ? s.y : 0.f;
+      S[(e + 2) % E] = own ? s.z : 0.f;
+      S[(e + 3) % E] = own ? s.w : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool own = col_on && i0 + e < ns;
+      const float s = S_at[own ? (size_t)col * ns + i0 + e : 0];
+      S[e] = own ? s : 0.f;
+    }
   }
   const T* xbc = (const T*)A.xbc;
   const T* dtp = (const T*)A.dt;
@@ -190,9 +204,16 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(SsmArgs A) {
       }
     }
   }
+  if (wide) {
 #pragma unroll
-  for (int e = 0; e < E; ++e)
-    if (col_on && i0 + e < ns) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
+    for (int e = 0; e < E; e += 4)
+      if (col_on && i0 + e < ns)
+        *reinterpret_cast<float4*>(S_at + (size_t)col * ns + i0 + e) = make_float4(S[e], S[(e + 1) % E], S[(e + 2) % E], S[(e + 3) % E]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (col_on && i0 + e < ns) S_at[(size_t)col * ns + i0 + e] = S[e];
+  }
 }
 
 extern "C" int jllm_ssm_scan(const void* xbc, int ld, const void* dt, int ldt, int dt_off, int dtype, const void* a_log,

@@ -1322,7 +1322,7 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a
                 state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor, n_requests: int, heads: int,
                 kv_heads: int, dk: int, dv: int, decay_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The gated delta rule over the step's rows, request by request and token by token, from and into ``state``
-    [slots, heads, dk, dv] (fp32). ``qkv`` [T, kv_heads x dk | kv_heads x dk | heads x dv] are the convolved q, k, v;
+    [slots, heads, dv, dk] (fp32; a head's matrix S [dk, dv] column by column). ``qkv`` [T, kv_heads x dk | kv_heads x dk | heads x dv] are the convolved q, k, v;
     ``proj`` rows hold, at the given offsets, the inputs a and b of decay and write strength (heads each). Per head:
     q and k become unit vectors (q also / sqrt(dk)); beta = sigmoid(b); g = exp(-exp(a_log) softplus(a + dt_bias));
     S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Returns the raw o, fp32 [T, heads x dv]. With
@@ -1347,8 +1347,8 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a
     if a_log.numel() != heads or dt_bias.numel() != (heads * dk if channel else heads):
         raise KernelError(f"a_log must have {heads} entries, dt_bias {heads * dk if channel else heads}")
     wd = _same_type("a_log and dt_bias", a_log, dt_bias)
-    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dk, dv):
-        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dk}, {dv}] tensor")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dv, dk):
+        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dv}, {dk}] tensor")
     _i32(row_req, T, "row -> request map")
     _i32(state_slots, n_requests, "state slots")
     out = torch.empty((T, heads * dv), dtype=torch.float32, device=qkv.device)
@@ -1383,7 +1383,7 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, a_log: torch.Te
              state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor, n_requests: int, heads: int, groups: int,
              n: int, dv: int) -> torch.Tensor:
     """A selective state-space recurrence over the step's rows, request by request and token by token, from and into
-    ``state`` [slots, heads, n, dv] (fp32). ``xbc`` [T, heads x dv | groups x n | groups x n] are the convolved x, B, C;
+    ``state`` [slots, heads, dv, n] (fp32; a head's matrix S [n, dv] column by column). ``xbc`` [T, heads x dv | groups x n | groups x n] are the convolved x, B, C;
     ``proj`` rows hold the step sizes' input (heads entries) from ``dt_off`` on. Per head (its group's B and C):
     dt = softplus(dt_in + dt_bias); S <- exp(-exp(a_log) dt) S + dt B x^T; y = S^T C + skip x. Returns y, fp32
     [T, heads x dv]."""
@@ -1400,8 +1400,8 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, a_log: torch.Te
     if a_log.numel() != heads or dt_bias.numel() != heads or skip.numel() != heads:
         raise KernelError(f"a_log, dt_bias and the skip weights must have {heads} entries")
     wd = _same_type("a_log, dt_bias and the skip weights", a_log, dt_bias, skip)
-    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, n, dv):
-        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {n}, {dv}] tensor")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dv, n):
+        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dv}, {n}] tensor")
     _i32(row_req, T, "row -> request map")
     _i32(state_slots, n_requests, "state slots")
     out = torch.empty((T, heads * dv), dtype=torch.float32, device=xbc.device)

@@ -1,6 +1,6 @@
 """A gated delta rule with short convolutions: a recurrent mixer whose per-request state has a fixed size.
 
-Per head the state is a matrix S [dim, vdim] in fp32; per token it decays, is corrected along the token's key towards
+Per head the state is a matrix S [dim, vdim] in fp32 (kept column by column, [vdim, dim]); per token it decays, is corrected along the token's key towards
 the token's value (the delta rule) and is read with the token's query. Beside it the state holds the last conv - 1
 inputs of the convolutions in front of q, k and v. Both live in the cache manager's state slots (one row per live
 request), so nothing grows with the context and nothing is paged.
@@ -110,7 +110,7 @@ class GatedDelta(Part):
 
     def state_spec(self):
         s = self.spec
-        return (StateSpec((s.heads, s.dim, s.vdim), torch.float32),
+        return (StateSpec((s.heads, s.vdim, s.dim), torch.float32),
                 StateSpec((max(s.conv - 1, 1), self.channels), torch.float32))
 
     def input_projection(self):

@@ -1,6 +1,6 @@
 """A selective state-space mixer (the Mamba-2 form): a recurrent mixer whose per-request state has a fixed size.
 
-Per head the state is a matrix S [state, vdim] in fp32; per token it decays by one number, takes in the outer product of
+Per head the state is a matrix S [state, vdim] in fp32 (kept column by column, [vdim, state]); per token it decays by one number, takes in the outer product of
 the token's B and x scaled by the step size, and is read with the token's C. Beside it the state holds the last conv - 1
 inputs of the convolution in front of x, B and C. Both live in the cache manager's state slots (one row per live
 request), so nothing grows with the context and nothing is paged.
@@ -70,7 +70,7 @@ class StateSpace(Part):
 
     def state_spec(self):
         s = self.spec
-        return (StateSpec((s.heads, s.state, s.vdim), torch.float32),
+        return (StateSpec((s.heads, s.vdim, s.state), torch.float32),
                 StateSpec((max(s.conv - 1, 1), self.channels), torch.float32))
 
     def heads_rows(self, xb, step, slot):

@@ -332,7 +332,7 @@ def test_delta_rule_recalls_a_far_memory(dtype, H, G, dk, dv):
     dev = lambda t: t.to(DEV)
     results = []
     for cuts in ([300, 2, 1, 1, 296], [T]):
-        state = torch.zeros(5, H, dk, dv, device=DEV)
+        state = torch.zeros(5, H, dv, dk, device=DEV)
         slots = torch.tensor([3, 1], dtype=torch.int32, device=DEV)
         got = [[], []]
         at = 0

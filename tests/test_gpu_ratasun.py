@@ -285,7 +285,7 @@ def test_channel_delta_recalls_a_far_memory(dtype, H, G, dk, dv):
     dev = lambda t: t.to(DEV)
     results = []
     for cuts in ([300, 2, 1, 1, 296], [T]):
-        state = torch.zeros(5, H, dk, dv, device=DEV)
+        state = torch.zeros(5, H, dv, dk, device=DEV)
         slots = torch.tensor([3, 1], dtype=torch.int32, device=DEV)
         got = [[], []]
         at = 0
@@ -365,7 +365,7 @@ def test_state_space_scan_recalls_a_far_memory(dtype, H, G, N, Pd):
     dev = lambda t: t.to(DEV)
     results = []
     for cuts in ([300, 2, 1, 1, 296], [T]):
-        state = torch.zeros(5, H, N, Pd, device=DEV)
+        state = torch.zeros(5, H, Pd, N, device=DEV)
         slots = torch.tensor([3, 1], dtype=torch.int32, device=DEV)
         got = [[], []]
         at = 0

@@ -65,7 +65,7 @@ def test_every_run_of_a_looped_layer_has_pages_and_state_of_its_own():
     # attention runs keep no state; a parallel run keeps the matrix per head and the convolutions' last inputs
     assert [p.state is None for p in plans] == [True, False, True, False, True, False, False]
     matrix, tail = plans[1].state
-    assert matrix.shape == (4, 12, 8) and tail.shape == (2, 2 * 2 * 12 + 4 * 8) and matrix.dtype == torch.float32
+    assert matrix.shape == (4, 8, 12) and tail.shape == (2, 2 * 2 * 12 + 4 * 8) and matrix.dtype == torch.float32
     cm = CacheManager(plans, 8, 256, 3, allocate=False)
     # the two runs of layer 1 share a page spec (one group, two of its runs), and so do the two runs of layer 2
     runs = sorted(tuple(g.runs) for g in cm.groups)

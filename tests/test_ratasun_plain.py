@@ -82,9 +82,9 @@ def test_every_run_of_a_looped_layer_has_pages_and_state_of_its_own():
     assert [p.kv is not None for p in plans] == [False, True, False, True, False, True, False, True, False]
     assert [p.state is not None for p in plans] == [True, False, True, False, True, False, True, False, True]
     matrix, tail = plans[0].state  # the delta rule: S per head, the last conv - 1 inputs of q | k | v
-    assert matrix.shape == (4, 12, 8) and tail.shape == (2, 2 * 2 * 12 + 4 * 8) and matrix.dtype == torch.float32
+    assert matrix.shape == (4, 8, 12) and tail.shape == (2, 2 * 2 * 12 + 4 * 8) and matrix.dtype == torch.float32
     matrix, tail = plans[2].state  # the state-space layer: S per head, the last conv - 1 inputs of x | B | C
-    assert matrix.shape == (6, 12, 8) and tail.shape == (3, 6 * 8 + 2 * 3 * 12) and tail.dtype == torch.float32
+    assert matrix.shape == (6, 8, 12) and tail.shape == (3, 6 * 8 + 2 * 3 * 12) and tail.dtype == torch.float32
     cm = CacheManager(plans, 8, 256, 3, allocate=False)
     runs = sorted(tuple(g.runs) for g in cm.groups)
     assert (1, 3, 5) in runs, "the three passes of layer 1 have pages of their own of one kind"
