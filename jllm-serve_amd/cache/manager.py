@@ -57,6 +57,7 @@ class PageSpec:
 
     rows: Tuple[CacheRow, ...]
     window: int = 0  # 0 = all earlier positions stay visible
+    keep_first: int = 0  # with a window: the positions before this one stay visible too, and their pages are never given back
 
     def __post_init__(self):
         names = [r.name for r in self.rows]
@@ -341,7 +342,8 @@ class CacheManager:
                 continue
             first = self._first_needed(g, rc.length)
             whole = first // self.page_size  # table entries wholly before `first`
-            for b in range(rc.released[gi], whole):
+            kept = -(-g.spec.keep_first // self.page_size)  # the pages of the kept first positions stay
+            for b in range(max(rc.released[gi], kept), whole):
                 p = rc.tables[gi][b]
                 if p >= 0:
                     g.pool.release(p)
@@ -359,7 +361,8 @@ class CacheManager:
             raise ValueError("a model with per-request state cannot be rewound")
         keep = -(-length // self.page_size)
         for gi, g in enumerate(self.groups):
-            if g.spec.window > 0 and self._first_needed(g, length) < rc.released[gi] * self.page_size:
+            kept = -(-g.spec.keep_first // self.page_size)
+            if g.spec.window > 0 and max(self._first_needed(g, length) // self.page_size, kept) < rc.released[gi]:
                 raise ValueError("the window of this group has already given back pages the shorter sequence needs")
             while len(rc.tables[gi]) > keep:
                 p = rc.tables[gi].pop()

@@ -56,6 +56,16 @@ class RopeSpec:
             raise ConfigError(f"invalid rope table: rotary_dim={self.rotary_dim} theta={self.theta}")
 
 
+@dataclass(frozen=True)
+class LearnedPositionSpec:
+    """A learned vector per position, added (unscaled) to the embedded rows at the input: row p of the tensor ``name``
+    [``rows``, hidden]. It rotates nothing in the mixers."""
+
+    name: str
+    rows: int
+    kind: str = "learned_position"
+
+
 # --------------------------------------------------------------------------- norms
 
 
@@ -76,6 +86,17 @@ class LayerNormSpec:
     bias_suffix: str = ".b"
     bias: bool = True
     kind: str = "layernorm"
+
+
+@dataclass(frozen=True)
+class DynTanhSpec:
+    """Dynamic Tanh, a norm without statistics: tanh(alpha * x) * w + b element by element, with a scalar ``alpha`` and a
+    vector ``b`` stored beside the weight under the weight's name with ``alpha_suffix`` / ``bias_suffix``. No mean, no
+    variance, no eps."""
+
+    bias_suffix: str = ".b"
+    alpha_suffix: str = ".alpha"
+    kind: str = "dyntanh"
 
 
 # --------------------------------------------------------------------------- mixers
@@ -198,6 +219,7 @@ class WideAttentionNames:
     norm_suffix: str = ".norm"
     lambda_q: Tuple[str, ...] = ("lq1", "lq2")  # differential attention: the vectors whose products give lambda
     lambda_k: Tuple[str, ...] = ("lk1", "lk2")
+    sink: str = "sink"
 
 
 @dataclass(frozen=True)
@@ -211,7 +233,13 @@ class WideAttentionSpec:
     projection before the heads are split. ``position``: index of a rotary table (applied with its pairing on the
     first rotary_dim entries of every head) or None. ``softcap`` > 0: scores become softcap * tanh(score / softcap).
     ``q_temp_every`` > 0: q at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1).
-    ``out_gate``: the concatenated heads are multiplied by sigmoid(W_g h) before the output product."""
+    ``out_gate``: the concatenated heads are multiplied by sigmoid(W_g h) before the output product; ``gate_per_head``:
+    W_g has one row per head and a head's whole output is multiplied by its one number. ``qk_norm`` "head": RMS norm of
+    every q head and every k head alone, with one gain vector [dim] for all q heads and one for all k heads (the
+    tensors ``<q>.norm`` / ``<k>.norm``). ``window`` > 0: the query at p sees keys p + 1 - window .. p, and, with
+    ``keep_first``, also the keys at positions before ``keep_first`` (which keep their true positions). ``sink``: a
+    learned number per head (tensor ``sink`` [heads]) whose exponential joins the softmax's denominator; it has no key
+    and no value and is not scaled."""
 
     heads: int
     kv_heads: int
@@ -229,6 +257,9 @@ class WideAttentionSpec:
     bias: bool = True
     out_gate: bool = True
     window: int = 0
+    keep_first: int = 0
+    sink: bool = False
+    gate_per_head: bool = False
     names: WideAttentionNames = WideAttentionNames()
     kind: str = "wide_attention"
 
@@ -398,6 +429,7 @@ class RoutedMoeNames:
     down: str = "down"
     router: str = "mlp.router"
     correction: str = "mlp.correction"
+    shared_gate: str = "mlp.shared.sg"
     ending: str = ""
 
 
@@ -407,7 +439,12 @@ class RoutedMoeSpec:
     scores are s + correction (``correction`` False: s alone); the experts form ``groups`` equal groups of neighbours, a
     group's score is the sum of its two largest choice scores, and only experts of the ``keep`` best groups can be
     chosen; the ``top`` largest choice scores win; their weights are their s divided by the sum (+ 1e-20) times
-    ``scale``. Experts are gated feed-forwards of ``hidden`` with the gate function ``activation``."""
+    ``scale``. Experts are gated feed-forwards of ``hidden`` with the gate function ``activation`` (and its ``limit``
+    where it has one). ``score`` "softmax": s = softmax(W_router h) over all experts. ``group_score`` "max": a group's
+    score is its largest choice score. ``normalize`` False: the weights are the chosen s times ``scale``, not divided by
+    their sum. ``shared`` (a GatedMlpSpec or None): a feed-forward that runs for every token and is added; with
+    ``shared_gate`` it is first multiplied by sigmoid(W_sg h), one number per token (tensor ``shared_gate`` [1,
+    hidden])."""
 
     experts: int
     top: int
@@ -417,6 +454,12 @@ class RoutedMoeSpec:
     keep: int = 1
     correction: bool = True
     activation: str = "silu"
+    limit: float = 0.0
+    score: str = "sigmoid"
+    group_score: str = "top2"
+    normalize: bool = True
+    shared: Any = None
+    shared_gate: bool = False
     names: RoutedMoeNames = RoutedMoeNames()
     kind: str = "routed_moe"
 
@@ -447,6 +490,11 @@ class LayerSpec:
     norm_mixer_out_name: str = ""
     norm_ffn_out_name: str = ""
     mixer_prefix: str = ""  # under the layer's prefix, for mixers whose tensor names are relative to it
+    # arrangement "hyper": the stream has ``streams`` copies per row; sublayer q reads u = sum_s in[s] x_s, and all
+    # streams are rewritten at once, x_t <- sum_s mix[s, t] x_s + out[t] * sublayer(norm(u)), with the tensors
+    # ``<prefix>.<hyper_names[q]>.in`` [streams], ``.out`` [streams], ``.mix`` [streams, streams] (indexed [from, to])
+    streams: int = 1
+    hyper_names: Tuple[str, str] = ("hc1", "hc2")
 
 
 @dataclass(frozen=True)
@@ -488,6 +536,7 @@ class ModelNames:
     embed: str = "model.embed_tokens.weight"
     final_norm: str = "model.norm.weight"
     head: str = "lm_head.weight"
+    embed_norm: str = ""  # the weight of a norm over the embedding output (ModelConfig.embed_norm)
 
 
 @dataclass(frozen=True)
@@ -508,6 +557,8 @@ class ModelConfig:
     max_positions: int = 4096
     embed_scale: float = 1.0
     logit_scale: float = 1.0  # the logits are the head's product times this
+    embed_norm: Any = None  # a norm spec: the embedded rows (with what the position encodings add) pass it first
+    streams: int = 1  # residual streams per row: all start as the embedding output, the final norm reads their sum
     description: str = ""
     names: ModelNames = ModelNames()
     raw: Mapping[str, Any] = field(default_factory=dict, compare=False, repr=False)

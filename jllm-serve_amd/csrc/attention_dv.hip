@@ -32,7 +32,7 @@ __global__ __launch_bounds__(PREP_THREADS) void qkv_prepare_kernel(
     T* __restrict__ qkv, int ld, const int* __restrict__ positions, const int* __restrict__ slots, int q_slots, int k_slots,
     int v_heads, int dk, int dv, const TG* __restrict__ gq, const TG* __restrict__ gk, float eps,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot_dims, float temp_coef, int temp_every,
-    T* __restrict__ kcache, T* __restrict__ vcache, int page_size) {
+    T* __restrict__ kcache, T* __restrict__ vcache, int page_size, int norm_per_head, int pair_halves) {
   extern __shared__ float sm[];  // q and k of the row
   __shared__ float red[PREP_THREADS / 64];
   const int t = blockIdx.x;
@@ -41,7 +41,18 @@ __global__ __launch_bounds__(PREP_THREADS) void qkv_prepare_kernel(
   const int pos = positions[t];
   for (int i = threadIdx.x; i < nq + nk; i += PREP_THREADS) sm[i] = ldf(row, i);
   __syncthreads();
-  if (gq) {  // the norm over a whole projection, before the heads are split
+  if (gq && norm_per_head) {  // every head alone, a wave per head; the gains [dk] are shared by the heads of q (of k)
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int head = wave; head < q_slots + k_slots; head += PREP_THREADS / 64) {
+      float* p = sm + (size_t)head * dk;
+      float ss = 0.f;
+      for (int i = lane; i < dk; i += 64) ss = fmaf(p[i], p[i], ss);
+      const float r = norm_scale(wave_sum(ss), dk, eps);
+      const TG* g = head < q_slots ? gq : gk;
+      for (int i = lane; i < dk; i += 64) p[i] = p[i] * r * ldf(g, i);
+    }
+    __syncthreads();
+  } else if (gq) {  // the norm over a whole projection, before the heads are split
     float sq = 0.f, sk = 0.f;
     for (int i = threadIdx.x; i < nq; i += PREP_THREADS) sq = fmaf(sm[i], sm[i], sq);
     for (int i = threadIdx.x; i < nk; i += PREP_THREADS) sk = fmaf(sm[nq + i], sm[nq + i], sk);
@@ -56,11 +67,12 @@ __global__ __launch_bounds__(PREP_THREADS) void qkv_prepare_kernel(
     const int pairs = (q_slots + k_slots) * half;
     for (int i = threadIdx.x; i < pairs; i += PREP_THREADS) {
       const int head = i / half, f = i % half;
-      float* p = sm + (size_t)head * dk + 2 * f;
+      float* p = sm + (size_t)head * dk + (pair_halves ? f : 2 * f);
+      const int other = pair_halves ? half : 1;  // the pair (f, f + half) or (2f, 2f + 1)
       const float c = cos_t[(size_t)pos * half + f], s = sin_t[(size_t)pos * half + f];
-      const float u = p[0], v = p[1];
+      const float u = p[0], v = p[other];
       p[0] = u * c - v * s;
-      p[1] = v * c + u * s;
+      p[other] = v * c + u * s;
     }
     __syncthreads();
   }
@@ -84,7 +96,7 @@ extern "C" int jllm_qkv_prepare(void* qkv, int ld, int dtype, int n_tokens, cons
                                 int q_slots, int k_slots, int v_heads, int dk, int dv, const void* gq, const void* gk,
                                 int gain_dtype, float eps, const float* cos_t, const float* sin_t, int rot_dims,
                                 float temp_coef, int temp_every, void* kcache, void* vcache, int page_size,
-                                hipStream_t stream) {
+                                int norm_per_head, int pair_halves, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (q_slots <= 0 || k_slots <= 0 || v_heads <= 0 || dk <= 0 || dv <= 0) JLLM_FAIL("qkv_prepare: sizes %d %d %d %d %d", q_slots, k_slots, v_heads, dk, dv);
   if (ld < (q_slots + k_slots) * dk + v_heads * dv) JLLM_FAIL("qkv_prepare: rows of %d entries are shorter than q, k and v", ld);
@@ -97,7 +109,7 @@ extern "C" int jllm_qkv_prepare(void* qkv, int ld, int dtype, int n_tokens, cons
     JLLM_DISPATCH_1(gain_dtype, TG, {
       qkv_prepare_kernel<T, TG><<<n_tokens, PREP_THREADS, smem, stream>>>(
           (T*)qkv, ld, positions, slots, q_slots, k_slots, v_heads, dk, dv, (const TG*)gq, (const TG*)gk, eps, cos_t, sin_t,
-          rot_dims, temp_coef, temp_every, (T*)kcache, (T*)vcache, page_size);
+          rot_dims, temp_coef, temp_every, (T*)kcache, (T*)vcache, page_size, norm_per_head, pair_halves);
     })
   })
   JLLM_CHECK_LAUNCH("qkv_prepare");
@@ -111,7 +123,7 @@ __global__ __launch_bounds__(64 * ADV_WAVES) void attention_dv_generic_kernel(
     const T* __restrict__ q, int ldq, TO* __restrict__ out, int ldo, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ row_req,
     const int* __restrict__ positions, int q_slots, int maps, int per_kv, int dk, int dv, int page_size, int window,
-    float scale, float softcap) {
+    float scale, float softcap, int keep_first, const float* __restrict__ sinks) {
   extern __shared__ float smem[];
   float* qs = smem;       // dk
   float* mg = smem + dk;  // ADV_WAVES x (2 + dv)
@@ -130,11 +142,15 @@ __global__ __launch_bounds__(64 * ADV_WAVES) void attention_dv_generic_kernel(
 #pragma unroll
   for (int a = 0; a < ADV_MAX_ACC; ++a) acc[a] = 0.f;
   float m = -INFINITY, l = 0.f;
-  const int b_first = first >> 6;
+  // keys before `kept` stay visible whatever the window: then the walk starts at block 0 and passes over the blocks
+  // between the kept keys and the window (block c still belongs to wave c % 4)
+  const int kept = window > 0 ? min(keep_first, first) : 0;
+  const int b_first = kept > 0 ? 0 : first >> 6;
   for (int blk = b_first + ((wave - b_first) & (ADV_WAVES - 1)); blk * 64 <= pos; blk += ADV_WAVES) {
     const int c0 = blk * 64;
+    if (c0 + 63 < first && c0 >= kept) continue;
     const int kj = c0 + lane;
-    const bool valid = kj >= first && kj <= pos;
+    const bool valid = (kj >= first || kj < kept) && kj <= pos;
     float sc = -INFINITY;
     int page = 0, off = 0;
     if (valid) {
@@ -153,8 +169,9 @@ __global__ __launch_bounds__(64 * ADV_WAVES) void attention_dv_generic_kernel(
 #pragma unroll
     for (int a = 0; a < ADV_MAX_ACC; ++a) acc[a] *= alpha;
     m = m_new;
-    const int j0 = max(0, first - c0), j1 = min(63, pos - c0);
+    const int j0 = c0 < kept ? 0 : max(0, first - c0), j1 = min(63, pos - c0);
     for (int j = j0; j <= j1; ++j) {  // the block's values in ascending order of the keys
+      if (c0 + j < first && c0 + j >= kept) continue;  // between the kept keys and the window: its page may be gone
       const float pj = __shfl(p, j, 64);
       const int pg = __shfl(page, j, 64), of = __shfl(off, j, 64);
       const T* vr = vcache + (((size_t)pg * v_heads + vh) * page_size + of) * dv;
@@ -191,6 +208,7 @@ __global__ __launch_bounds__(64 * ADV_WAVES) void attention_dv_generic_kernel(
     }
     m = m_new;
   }
+  if (sinks) l += expf(sinks[s / maps] - m);  // one more term of the denominator, with no value
   const float inv = 1.0f / l;
   TO* o = out + (size_t)t * ldo + (size_t)s * dv;
 #pragma unroll
@@ -205,13 +223,13 @@ extern "C" int jllm_attention_dv_generic(const void* q, int ldq, int dtype, void
                                          const void* kcache, const void* vcache, const int* block_table, int max_blocks,
                                          const int* row_req, const int* positions, int n_tokens, int heads, int kv_heads,
                                          int maps, int dk, int dv, int page_size, int window, float scale, float softcap,
-                                         hipStream_t stream) {
+                                         int keep_first, const float* sinks, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || maps <= 0) JLLM_FAIL("attention: %d query heads over %d kv heads with %d maps", heads, kv_heads, maps);
   if (dk <= 0 || dv <= 0 || dv > 64 * ADV_MAX_ACC || dk > 4096) JLLM_FAIL("attention: key size %d, value size %d (this kernel takes values up to %d)", dk, dv, 64 * ADV_MAX_ACC);
   const int q_slots = heads * maps;
   if (q_slots > 65535) JLLM_FAIL("attention: too many heads");
-  if (page_size <= 0 || max_blocks <= 0 || window < 0) JLLM_FAIL("attention: page_size %d max_blocks %d window %d", page_size, max_blocks, window);
+  if (page_size <= 0 || max_blocks <= 0 || window < 0 || keep_first < 0) JLLM_FAIL("attention: page_size %d max_blocks %d window %d, %d first keys kept", page_size, max_blocks, window, keep_first);
   if (ldq < q_slots * dk || ldo < q_slots * dv) JLLM_FAIL("attention: row strides %d/%d", ldq, ldo);
   dim3 grid(n_tokens, q_slots);
   const size_t smem = (size_t)(dk + ADV_WAVES * (2 + dv)) * sizeof(float);
@@ -219,7 +237,7 @@ extern "C" int jllm_attention_dv_generic(const void* q, int ldq, int dtype, void
     JLLM_DISPATCH_1(out_dtype, TO, {
       attention_dv_generic_kernel<T, TO><<<grid, 64 * ADV_WAVES, smem, stream>>>(
           (const T*)q, ldq, (TO*)out, ldo, (const T*)kcache, (const T*)vcache, block_table, max_blocks, row_req, positions,
-          q_slots, maps, maps * (heads / kv_heads), dk, dv, page_size, window, scale, softcap);
+          q_slots, maps, maps * (heads / kv_heads), dk, dv, page_size, window, scale, softcap, keep_first, sinks);
     })
   })
   JLLM_CHECK_LAUNCH("attention_dv_generic");
@@ -232,7 +250,8 @@ template <typename TA, typename TG, typename TW, typename TO>
 __global__ __launch_bounds__(64) void heads_finish_kernel(const TA* __restrict__ att, int lda, int maps, int dv,
                                                           float lambda, int normed, float eps, float norm_mul,
                                                           const TW* __restrict__ gain, const TG* __restrict__ gate, int ldg,
-                                                          int gate_fn, float out_mul, TO* __restrict__ out, int ldo) {
+                                                          int gate_fn, float out_mul, TO* __restrict__ out, int ldo,
+                                                          int gate_per_head) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const TA* a = att + (size_t)t * lda + (size_t)h * maps * dv;
   float ss = 0.f;
@@ -251,21 +270,22 @@ __global__ __launch_bounds__(64) void heads_finish_kernel(const TA* __restrict__
     o *= r;
     if (gain) o *= ldf(gain, j);
     if (gate) {
-      const float z = ldf(gate + (size_t)t * ldg, (size_t)h * dv + j);
+      const float z = ldf(gate + (size_t)t * ldg, gate_per_head ? (size_t)h : (size_t)h * dv + j);
       o *= (gate_fn == 1 ? z : 1.0f) / (1.0f + expf(-z));  // 0: sigmoid(z), 1: silu(z)
     }
     stf(out + (size_t)t * ldo, (size_t)h * dv + j, o * out_mul);
   }
 }
 
-// att [rows, lda]: heads x maps x dv per row; gate [rows, ldg]: heads x dv per row or null; out [rows, ldo]
+// att [rows, lda]: heads x maps x dv per row; gate [rows, ldg]: heads x dv per row (`gate_per_head`: heads per row, one
+// number for the whole head) or null; out [rows, ldo]
 extern "C" int jllm_heads_finish(const void* att, int lda, int att_dtype, int n_tokens, int heads, int maps, int dv,
                                  float lambda, int normed, float eps, float norm_mul, const void* gain, int gain_dtype,
                                  const void* gate, int ldg, int gate_dtype, int gate_fn, float out_mul, void* out, int ldo, int out_dtype,
-                                 hipStream_t stream) {
+                                 int gate_per_head, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (heads <= 0 || heads > 65535 || dv <= 0 || (maps != 1 && maps != 2)) JLLM_FAIL("heads_finish: %d heads of %d with %d maps (one or two are taken)", heads, dv, maps);
-  if (lda < heads * maps * dv || ldo < heads * dv || (gate && ldg < heads * dv)) JLLM_FAIL("heads_finish: short rows");
+  if (lda < heads * maps * dv || ldo < heads * dv || (gate && ldg < (gate_per_head ? heads : heads * dv))) JLLM_FAIL("heads_finish: short rows");
   if (gate_fn != 0 && gate_fn != 1) JLLM_FAIL("heads_finish: gate function %d (0 sigmoid and 1 silu are built)", gate_fn);
   dim3 grid(n_tokens, heads);
   JLLM_DISPATCH_1(att_dtype, TA, {
@@ -273,7 +293,8 @@ extern "C" int jllm_heads_finish(const void* att, int lda, int att_dtype, int n_
       JLLM_DISPATCH_1(gain_dtype, TW, {
         JLLM_DISPATCH_1(out_dtype, TO, {
           heads_finish_kernel<TA, TG, TW, TO><<<grid, 64, 0, stream>>>((const TA*)att, lda, maps, dv, lambda, normed, eps, norm_mul,
-                                                                      (const TW*)gain, (const TG*)gate, ldg, gate_fn, out_mul, (TO*)out, ldo);
+                                                                      (const TW*)gain, (const TG*)gate, ldg, gate_fn, out_mul, (TO*)out, ldo,
+                                                                      gate_per_head);
         })
       })
     })
@@ -291,7 +312,7 @@ __global__ __launch_bounds__(64) void heads_finish_split_kernel(const float* __r
                                                                 int dv, float lambda, int normed, float eps, float norm_mul,
                                                                 const TW* __restrict__ gain, const TG* __restrict__ gate,
                                                                 int ldg, int gate_fn, float out_mul, TO* __restrict__ out,
-                                                                int ldo) {
+                                                                int ldo, int gate_per_head, const float* __restrict__ sinks) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   float o[4] = {0.f, 0.f, 0.f, 0.f};  // dv <= 256
   for (int m = 0; m < maps; ++m) {
@@ -300,7 +321,9 @@ __global__ __launch_bounds__(64) void heads_finish_split_kernel(const float* __r
     const float lz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
     const float mx = wave_max(mz);
     const float wz = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);
-    const float inv = 1.0f / wave_sum(lz * wz);
+    // a sink is one more term of the denominator: exp(sink) on the scale of the ranges' common maximum
+    const float sink_term = sinks ? __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - mx) : 0.f;
+    const float inv = 1.0f / (wave_sum(lz * wz) + sink_term);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int j = lane + 64 * jj;
@@ -330,7 +353,7 @@ __global__ __launch_bounds__(64) void heads_finish_split_kernel(const float* __r
     float v = o[jj] * r;
     if (gain) v *= ldf(gain, j);
     if (gate) {
-      const float z = ldf(gate + (size_t)t * ldg, (size_t)h * dv + j);
+      const float z = ldf(gate + (size_t)t * ldg, gate_per_head ? (size_t)h : (size_t)h * dv + j);
       v *= (gate_fn == 1 ? z : 1.0f) / (1.0f + expf(-z));
     }
     stf(out + (size_t)t * ldo, (size_t)h * dv + j, v * out_mul);
@@ -340,19 +363,20 @@ __global__ __launch_bounds__(64) void heads_finish_split_kernel(const float* __r
 extern "C" int jllm_heads_finish_split(const float* partial, int splits, int n_tokens, int heads, int maps, int dv, float lambda,
                                        int normed, float eps, float norm_mul, const void* gain, int gain_dtype, const void* gate,
                                        int ldg, int gate_dtype, int gate_fn, float out_mul, void* out, int ldo, int out_dtype,
-                                       hipStream_t stream) {
+                                       int gate_per_head, const float* sinks, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (heads <= 0 || heads > 65535 || dv <= 0 || dv > 256 || (maps != 1 && maps != 2) || splits < 1 || splits > 64)
     JLLM_FAIL("heads_finish: %d heads of %d with %d maps in %d key ranges", heads, dv, maps, splits);
-  if (ldo < heads * dv || (gate && ldg < heads * dv)) JLLM_FAIL("heads_finish: short rows");
+  if (ldo < heads * dv || (gate && ldg < (gate_per_head ? heads : heads * dv))) JLLM_FAIL("heads_finish: short rows");
   if (gate_fn != 0 && gate_fn != 1) JLLM_FAIL("heads_finish: gate function %d (0 sigmoid and 1 silu are built)", gate_fn);
+  if (sinks && maps != 1) JLLM_FAIL("heads_finish: a sink with %d maps per head", maps);
   dim3 grid(n_tokens, heads);
   JLLM_DISPATCH_1(gate_dtype, TG, {
     JLLM_DISPATCH_1(gain_dtype, TW, {
       JLLM_DISPATCH_1(out_dtype, TO, {
         heads_finish_split_kernel<TG, TW, TO><<<grid, 64, 0, stream>>>(partial, splits, maps, dv, lambda, normed, eps, norm_mul,
                                                                       (const TW*)gain, (const TG*)gate, ldg, gate_fn, out_mul,
-                                                                      (TO*)out, ldo);
+                                                                      (TO*)out, ldo, gate_per_head, sinks);
       })
     })
   })

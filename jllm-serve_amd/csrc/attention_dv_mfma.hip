@@ -33,7 +33,8 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     const bf16_t* __restrict__ q, int ldq, float* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
     const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ positions, int maps, int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window,
-    float scale, float softcap, float* __restrict__ partial, int per_split, int share, int q_slots) {
+    float scale, float softcap, float* __restrict__ partial, int per_split, int share, int q_slots, int keep_first,
+    const float* __restrict__ sinks) {
   constexpr int DK = DK16 * 16;
   constexpr int DVP = DB * 32;
   constexpr int KLD = DK + 8;
@@ -74,11 +75,17 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
 #pragma unroll
     for (int i = 0; i < DK16; ++i) qf[i] = *(const u32x4*)(qr + i * 16);
   }
-  int kt_first = (k_lo / AT_KEYS) * AT_KEYS;
-  int n_blocks = (k_hi - kt_first) / AT_KEYS + 1;
+  // The blocks of a tile are numbered 0, 1, ...: first the blocks of the kept first keys that lie wholly before the
+  // window's first block (keys before `kept` stay visible whatever the window), then the window's blocks.
+  const int kept = window > 0 ? min(keep_first, k_lo) : 0;  // keys [0, kept) of the tile beside [k_lo, k_hi]
+  const int win_first = (k_lo / AT_KEYS) * AT_KEYS;
+  const int n_kept = min((kept + AT_KEYS - 1) / AT_KEYS, win_first / AT_KEYS);
+  int it_first = 0;
+  int n_blocks = n_kept + (k_hi - win_first) / AT_KEYS + 1;
+  auto block_keys = [&](int it) { return it < n_kept ? it * AT_KEYS : win_first + (it - n_kept) * AT_KEYS; };
   if (partial) {  // this workgroup's share of the tile's blocks
     const int b0 = blockIdx.z * per_split;
-    kt_first += b0 * AT_KEYS;
+    it_first = b0;
     n_blocks = min(per_split, n_blocks - b0);
     if (n_blocks <= 0) {  // nothing left for this split: it says so (the same for all threads: no barrier was met)
       if (lane_on && half == 0) {
@@ -97,13 +104,13 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     for (int j = 0; j < KCH; ++j) {
       const int c = tid + 256 * j;
       const int kabs = kt + c / (DK16 * 2);
-      kpg[j] = (c < AT_KEYS * DK16 * 2 && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+      kpg[j] = (c < AT_KEYS * DK16 * 2 && (kabs >= k_lo || kabs < kept) && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
     }
 #pragma unroll
     for (int j = 0; j < VCH; ++j) {
       const int c = tid + 256 * j;
       const int kabs = kt + c / VPC;
-      vpg[j] = (c < AT_KEYS * VPC && (c % VPC) * 8 < dv && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+      vpg[j] = (c < AT_KEYS * VPC && (c % VPC) * 8 < dv && (kabs >= k_lo || kabs < kept) && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
     }
   };
   auto load_block = [&](int kt) {
@@ -151,17 +158,19 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
   const float log2e = 1.4426950408889634f;
   const float sl = softcap > 0.f ? log2e : scale * log2e;  // capped scores are final; raw ones are scaled in the exponent
   const float cap_in = softcap > 0.f ? 2.0f * log2e * scale / softcap : 0.f;
-  load_pages(kt_first);
-  load_block(kt_first);
-  load_pages(kt_first + AT_KEYS);
+  // beyond a tile's last block the block numbers name keys past k_hi, whose table entries are never read
+  load_pages(block_keys(it_first));
+  load_block(block_keys(it_first));
+  load_pages(block_keys(it_first + 1));
   store_block(0);
   __syncthreads();
   int buf = 0;
-  for (int it = 0, kt = kt_first; it < n_blocks; ++it, kt += AT_KEYS, buf ^= 1) {
+  for (int it = 0; it < n_blocks; ++it, buf ^= 1) {
+    const int kt = block_keys(it_first + it);
     const bool more = it + 1 < n_blocks;
     if (more) {
-      load_block(kt + AT_KEYS);
-      load_pages(kt + 2 * AT_KEYS);
+      load_block(block_keys(it_first + it + 1));
+      load_pages(block_keys(it_first + it + 2));
     }
     if (wave_on && kt <= wave_hi) {
       const bf16_t* Kb = Ks + buf * KSZ;
@@ -182,7 +191,7 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
           for (int e = 0; e < 16; ++e)
             sc[kb][e] = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sc[kb][e] * cap_in)));
       }
-      const bool all_visible = kt + AT_KEYS - 1 <= wave_lo_pos && kt >= wave_first;
+      const bool all_visible = kt + AT_KEYS - 1 <= wave_lo_pos && (kt >= wave_first || kt + AT_KEYS <= kept);
       if (!all_visible) {
         const int key0 = kt + half * 4;
 #pragma unroll
@@ -190,7 +199,7 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const int key = key0 + kb * 32 + 8 * (e >> 2) + (e & 3);
-            sc[kb][e] = (key >= first_q && key <= pos_q) ? sc[kb][e] : -INFINITY;
+            sc[kb][e] = ((key >= first_q || key < keep_first) && key <= pos_q) ? sc[kb][e] : -INFINITY;
           }
       }
       // the maximum of the scores as they enter the exponent (a negative scale turns the order round)
@@ -266,6 +275,8 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     }
     return;
   }
+  // a sink is one more term of the denominator, exp(sink), with no value; m is an exponent of two
+  if (sinks) l += __builtin_amdgcn_exp2f(sinks[s / maps] * log2e - m);
   const float inv = 1.0f / l;
   float* orow = out + (size_t)(row0 + wq) * ldo + (size_t)s * dv;
 #pragma unroll
@@ -281,14 +292,16 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
 // Lane z holds split z's maximum and sum (at most 64 splits), so the weights of all splits are known after two wave
 // reductions and the sums' loads are independent of each other.
 __global__ __launch_bounds__(64) void attention_dv_merge_kernel(const float* __restrict__ partial, int splits, int dv,
-                                                                float* __restrict__ out, int ldo) {
+                                                                float* __restrict__ out, int ldo, int maps,
+                                                                const float* __restrict__ sinks) {
   const int t = blockIdx.x, s = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + ((size_t)t * gridDim.y + s) * splits * (dv + 2);
   const float mz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv] : -INFINITY;
   const float lz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
   const float mx = wave_max(mz);
   const float wz = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);
-  const float inv = 1.0f / wave_sum(lz * wz);
+  const float sink_term = sinks ? __builtin_amdgcn_exp2f(sinks[s / maps] * 1.4426950408889634f - mx) : 0.f;
+  const float inv = 1.0f / (wave_sum(lz * wz) + sink_term);
   for (int d = lane; d < dv; d += 64) {
     float acc = 0.f;
 #pragma unroll 4
@@ -305,7 +318,7 @@ template <int DK16, int DB>
 static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq, float* out, int ldo, const bf16_t* kc,
                         const bf16_t* vc, const int* block_table, int max_blocks, const int* tiles, const int* positions, int maps,
                         int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window, float scale, float softcap,
-                        float* partial, int per_split, int share, int q_slots) {
+                        float* partial, int per_split, int share, int q_slots, int keep_first, const float* sinks) {
   const size_t smem = (size_t)2 * AT_KEYS * ((DK16 * 16 + 8) + (DB * 32 + 32)) * sizeof(bf16_t);
   static bool raised = false;
   if (smem > 64 * 1024 && !raised) {
@@ -315,7 +328,7 @@ static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq,
   }
   attention_dv_tiles_kernel<DK16, DB><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, block_table, max_blocks, tiles, positions,
                                                                  maps, per_kv, k_slots, v_heads, dv, page_shift, window, scale, softcap,
-                                                                 partial, per_split, share, q_slots);
+                                                                 partial, per_split, share, q_slots, keep_first, sinks);
   return 0;
 }
 
@@ -327,11 +340,11 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
                                       const int* block_table, int max_blocks, const int* tiles, int n_tiles,
                                       const int* positions, int heads, int kv_heads, int maps, int dk, int dv, int page_size,
                                       int window, float scale, float softcap, int splits, int per_split, float* partial,
-                                      int n_rows, int defer_merge, hipStream_t stream) {
+                                      int n_rows, int defer_merge, int keep_first, const float* sinks, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || maps <= 0) JLLM_FAIL("attention: %d query heads over %d kv heads with %d maps", heads, kv_heads, maps);
   if ((dk & 15) || dk < 16 || dk > 256 || (dv & 7) || dv < 8 || dv > 256) return 1;
-  if (!(scale > 0.f) || softcap < 0.f) return 1;  // the maximum is taken before the scale's sign could matter
+  if (!(scale > 0.f) || softcap < 0.f || keep_first < 0) return 1;  // the maximum is taken before the scale's sign could matter
   if ((ldq & 7) || (ldo & 3) || ((uintptr_t)q & 15) || ((uintptr_t)out & 15) || ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15)) return 1;
   if (page_size <= 0 || (page_size & (page_size - 1)) || n_tiles > 65535 || heads * maps > 65535) return 1;
   int page_shift = 0;
@@ -346,7 +359,7 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
   int rc = 1;
 #define AT_ARGS grid, stream, (const bf16_t*)q, ldq, out, ldo, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, max_blocks, \
                 tiles, positions, maps, per_kv, kv_heads * maps, kv_heads, dv, page_shift, window, scale, softcap, partial, per_split, \
-                share, q_slots
+                share, q_slots, keep_first, sinks
 #define AT_DB(N)                                  \
   switch (db) {                                   \
     case 1: rc = launch_tiles<N, 1>(AT_ARGS); break; \
@@ -370,7 +383,7 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
 #undef AT_ARGS
   if (rc < 0) JLLM_FAIL("attention: cannot reserve LDS");
   // `defer_merge`: the caller's next kernel reads the splits itself (heads_finish_split in attention_dv.hip)
-  if (partial && !defer_merge) attention_dv_merge_kernel<<<dim3(n_rows, q_slots), 64, 0, stream>>>(partial, splits, dv, out, ldo);
+  if (partial && !defer_merge) attention_dv_merge_kernel<<<dim3(n_rows, q_slots), 64, 0, stream>>>(partial, splits, dv, out, ldo, maps, sinks);
   JLLM_CHECK_LAUNCH("attention_dv_bf16");
   return 0;
 }

@@ -2,11 +2,12 @@
 // or table[t][0 .. top) where a router chose them for this step's rows (`tokens` null). Everything happens on the
 // device, so a step needs no answer from the GPU before it launches (and can be captured).
 //
-//   moe_router    one wave per row, from the router's fp32 logits z [T, E]: s = sigmoid(z); choice = s + correction;
-//                 the experts form `groups` equal groups of neighbours, a group's score is the sum of its two largest
-//                 choice scores and only the `keep` best groups can be chosen from; the `top` largest choice scores
-//                 among those win (the lowest index among equals); weights = s of the chosen / (their sum + 1e-20) *
-//                 scale. Writes the chosen experts [T, top] (int32) and their weights [T, top] (fp32)
+//   moe_router    one wave per row, from the router's fp32 logits z [T, E]: s = sigmoid(z) (or softmax(z) over all
+//                 experts); choice = s + correction; the experts form `groups` equal groups of neighbours, a group's
+//                 score is the sum of its two largest choice scores (or the largest) and only the `keep` best groups
+//                 can be chosen from; the `top` largest choice scores among those win (the lowest index among equals);
+//                 weights = s of the chosen / (their sum + 1e-20) * scale (or s * scale, not normalised). Writes the
+//                 chosen experts [T, top] (int32) and their weights [T, top] (fp32)
 //   moe_route     one workgroup: counts the assignments (row, k) of every expert, lays them out expert by expert in
 //                 `sorted`, and cuts each expert's run into tiles of at most `tile_rows` rows: tiles[i] = (expert,
 //                 first place in `sorted`, rows); the tiles no expert needs have 0 rows
@@ -16,7 +17,8 @@
 //                 and writes fp32 rows by assignment, or, with top = 1, adds them straight into the residual rows
 //   moe_combine   residual[t] += weight * sum_k y[t * top + k], k ascending (or y[place_of[t * top + k]] where the second
 //                 product wrote its rows in the order of `sorted`); with `weights` [T, top] every term has its own
-//                 factor weights[t, k] as well
+//                 factor weights[t, k] as well; a shared expert's fp32 rows may join the sum, times the sigmoid of a
+//                 gate logit per row
 //
 // The order of `sorted` within an expert comes from LDS atomics and may differ between runs; no result depends on it
 // (every output is one accumulator over ascending k of its own row and weight row). This file is the fp32 path
@@ -196,23 +198,32 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
 // ---------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
                                                          int top, float weight, const int* __restrict__ place_of,
-                                                         const float* __restrict__ weights) {
+                                                         const float* __restrict__ weights, const float* __restrict__ shared,
+                                                         const float* __restrict__ shared_gate, int ldsg, int overwrite) {
   const int t = blockIdx.x;
+  // a shared expert's rows join the sum, times sigmoid of the row's gate logit where it has one
+  const float sg = shared ? (shared_gate ? 1.0f / (1.0f + expf(-shared_gate[(size_t)t * ldsg])) : 1.0f) : 0.f;
   for (int i = threadIdx.x; i < width; i += 256) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) {
       const size_t row = place_of ? (size_t)place_of[t * top + k] : (size_t)t * top + k;
       s = weights ? fmaf(weights[(size_t)t * top + k], y[row * width + i], s) : s + y[row * width + i];
     }
-    residual[(size_t)t * width + i] += weight * s;
+    float r = overwrite ? 0.f : residual[(size_t)t * width + i];
+    if (shared) r = fmaf(sg, shared[(size_t)t * width + i], r);
+    residual[(size_t)t * width + i] = r + weight * s;
   }
 }
 
+// `shared` [T, width] fp32 (optional): one more term per row, times sigmoid(shared_gate[t * ldsg]) where a gate is given;
+// `overwrite`: the rows of `residual` are written, not added to (it may be the same tensor as `shared`)
 extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, const int* place_of,
-                                const float* weights, hipStream_t stream) {
+                                const float* weights, const float* shared, const float* shared_gate, int ldsg, int overwrite,
+                                hipStream_t stream) {
   if (T <= 0) return 0;
   if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights);
+  if (shared_gate && !shared) JLLM_FAIL("moe_combine: a gate without the shared rows it weighs");
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg, overwrite);
   JLLM_CHECK_LAUNCH("moe_combine");
   return 0;
 }
@@ -222,7 +233,8 @@ extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int widt
 template <typename TC>
 __global__ __launch_bounds__(64) void moe_router_kernel(const float* __restrict__ z, int ldz, const TC* __restrict__ correction,
                                                        int E, int groups, int keep, int top, float scale,
-                                                       int* __restrict__ chosen, float* __restrict__ weights) {
+                                                       int* __restrict__ chosen, float* __restrict__ weights, int softmax,
+                                                       int group_max, int normalize) {
   extern __shared__ float rs[];
   float* s = rs;
   float* choice = rs + E;
@@ -230,8 +242,16 @@ __global__ __launch_bounds__(64) void moe_router_kernel(const float* __restrict_
   int* allowed = (int*)(rs + 2 * E + groups);
   const int t = blockIdx.x, lane = threadIdx.x;
   const int per = E / groups;
+  float zmax = -INFINITY, zden = 1.0f;
+  if (softmax) {  // s = softmax(z) over all experts
+    for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, z[(size_t)t * ldz + e]);
+    zmax = wave_max(zmax);
+    float d = 0.f;
+    for (int e = lane; e < E; e += 64) d += expf(z[(size_t)t * ldz + e] - zmax);
+    zden = wave_sum(d);
+  }
   for (int e = lane; e < E; e += 64) {
-    const float v = 1.0f / (1.0f + expf(-z[(size_t)t * ldz + e]));
+    const float v = softmax ? expf(z[(size_t)t * ldz + e] - zmax) / zden : 1.0f / (1.0f + expf(-z[(size_t)t * ldz + e]));
     s[e] = v;
     choice[e] = v + (correction ? ldf(correction, e) : 0.f);
   }
@@ -242,7 +262,7 @@ __global__ __launch_bounds__(64) void moe_router_kernel(const float* __restrict_
       const float v = choice[g * per + i];
       if (v > a) b = a, a = v; else if (v > b) b = v;
     }
-    gscore[g] = per > 1 ? a + b : a;
+    gscore[g] = (per > 1 && !group_max) ? a + b : a;
     allowed[g] = 0;
   }
   __syncthreads();
@@ -283,11 +303,13 @@ __global__ __launch_bounds__(64) void moe_router_kernel(const float* __restrict_
     __syncthreads();
   }
   if (lane == 0)
-    for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = weights[(size_t)t * top + k] / (sum + 1e-20f) * scale;
+    for (int k = 0; k < top; ++k)
+      weights[(size_t)t * top + k] = normalize ? weights[(size_t)t * top + k] / (sum + 1e-20f) * scale : weights[(size_t)t * top + k] * scale;
 }
 
 extern "C" int jllm_moe_router(const float* z, int ldz, const void* correction, int c_dtype, int T, int E, int groups, int keep,
-                               int top, float scale, int* chosen, float* weights, hipStream_t stream) {
+                               int top, float scale, int* chosen, float* weights, int softmax, int group_max, int normalize,
+                               hipStream_t stream) {
   if (T <= 0) return 0;
   if (E <= 0 || top <= 0 || top > E || ldz < E) JLLM_FAIL("moe_router: top %d of %d experts in rows of %d", top, E, ldz);
   if (groups <= 0 || E % groups || keep <= 0 || keep > groups || keep * (E / groups) < top)
@@ -295,7 +317,8 @@ extern "C" int jllm_moe_router(const float* z, int ldz, const void* correction, 
   const size_t smem = (size_t)(2 * E + 2 * groups) * sizeof(float);
   if (smem > 64 * 1024) JLLM_FAIL("moe_router: %d experts are more than this kernel's LDS holds", E);
   JLLM_DISPATCH_1(c_dtype, TC, {
-    moe_router_kernel<TC><<<T, 64, smem, stream>>>(z, ldz, (const TC*)correction, E, groups, keep, top, scale, chosen, weights);
+    moe_router_kernel<TC><<<T, 64, smem, stream>>>(z, ldz, (const TC*)correction, E, groups, keep, top, scale, chosen, weights, softmax,
+                                                   group_max, normalize);
   })
   JLLM_CHECK_LAUNCH("moe_router");
   return 0;

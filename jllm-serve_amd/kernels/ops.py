@@ -73,17 +73,20 @@ def _declare(lib) -> None:
         "jllm_latent_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
         "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
         "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
-        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P, _P],
-        "jllm_moe_router": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P, _P, _P, _I, _I, _P],
+        "jllm_moe_router": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _I, _I, _I, _P],
+        "jllm_gather_add": [_P, _I, _P, _I, _I, _P, _I, _I, _P],
+        "jllm_dyntanh_read": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+        "jllm_streams_write": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
         "jllm_concat_rows": [_P, _P, _I, _I, _P, _I, _I, _P],
         "jllm_ssm_scan": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
         "jllm_gated_group_norm": [_P, _I, _P, _I, _I, _P, _I, _F, _I, _I, _I, _P, _I, _I, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
         "jllm_layernorm_seam": [_P, _P, _I, _I, _P, _I, _P, _I, _I, _F, _F, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _P],
-        "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
-        "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
-        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
-        "jllm_heads_finish_split": [_P, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
+        "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _I, _I, _P],
+        "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _P],
+        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _I, _P],
+        "jllm_heads_finish_split": [_P, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P],
         "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P],
         "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     }
@@ -118,7 +121,7 @@ _OPTIONAL_SIGS = {
     "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_gemm_mfma_grouped_bf16": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _I, _P],
-    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _I, _I, _P],
+    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _I, _I, _I, _P, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -234,6 +237,86 @@ def concat_rows(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype) -> tor
     n, d = a.shape
     out = activation_rows(n, 2 * d, out_dtype, a.device)
     _call("jllm_concat_rows", _ptr(a), _ptr(b), n, d, _ptr(out), _code(out_dtype), out.stride(0), _stream())
+    return out
+
+
+def gather_add(x: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """x[t, :] += table[ids[t], :] on fp32 rows (a learned table indexed by position, added at the input)."""
+    _dev(x, table, ids)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous() or table.dim() != 2 or not table.is_contiguous() \
+            or table.shape[1] != x.shape[1]:
+        raise KernelError("gather_add takes contiguous fp32 rows [n, width] and a table [rows, width]")
+    n = x.shape[0]
+    _i32(ids, n, "row indices")
+    _call("jllm_gather_add", _ptr(x), x.stride(0), _ptr(table), _code(table.dtype), table.shape[0], _ptr(ids), n, x.shape[1], _stream())
+
+
+MAX_STREAMS = 8   # residual streams per row that the stream kernels take (csrc/streams.hip)
+
+
+def _dyt(weight, bias, alpha, width):
+    for t in (weight, bias):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != width:
+            raise KernelError(f"the Dynamic-Tanh norm's weight and bias are contiguous fp32 tensors of {width} entries")
+    if alpha.dtype != torch.float32 or alpha.numel() != 1:
+        raise KernelError("the Dynamic-Tanh norm's slope is one fp32 number on the device")
+
+
+def dyntanh(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor, out_dtype: torch.dtype, *,
+            streams: int = 1, read: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+            copies: int = 1) -> torch.Tensor:
+    """tanh(alpha * u) * weight + bias, element by element, in ``out_dtype``: u is the fp32 row of ``x`` [n, width], or,
+    with ``read`` (fp32 [streams]), the weighted sum sum_s read[s] * x[t, s, :] of the row's streams (``x`` [n, streams x
+    width]). ``rows``: the input row of every output row; ``copies``: the result is written that many times side by side
+    (the start of several streams). No statistics of the row enter: the norm has no mean, variance or eps."""
+    _dev(x, weight, bias, alpha, read, rows)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous() or x.shape[1] % max(streams, 1):
+        raise KernelError("dyntanh takes contiguous fp32 rows [n, streams x width]")
+    width = x.shape[1] // streams
+    _dyt(weight, bias, alpha, width)
+    if not 1 <= streams <= MAX_STREAMS or (streams > 1 and read is None):
+        raise KernelError(f"dyntanh: {streams} streams (1..{MAX_STREAMS}, with their weights)")
+    if read is not None and (read.dtype != torch.float32 or not read.is_contiguous() or read.numel() != streams):
+        raise KernelError(f"dyntanh: the streams' weights are a contiguous fp32 tensor of {streams} entries")
+    n = x.shape[0] if rows is None else rows.numel()
+    _i32(rows, n, "row list")
+    out = activation_rows(n, copies * width, out_dtype, x.device) if copies == 1 else \
+        torch.empty((n, copies * width), dtype=out_dtype, device=x.device)
+    _call("jllm_dyntanh_read", _ptr(x), _ptr(rows), n, width, streams, _ptr(read), _ptr(weight), _ptr(bias), _ptr(alpha),
+          _ptr(out), _code(out_dtype), out.stride(0), int(copies), _stream())
+    return out
+
+
+def streams_write(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out_w: torch.Tensor, *, nxt=None,
+                  out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """All streams of every row at once from the old ones, in place on ``x`` fp32 [n, streams x width]:
+    new[r] = sum_s mix[s, r] * old[s] + out_w[r] * y (``y`` fp32 [n, width], a sublayer's output; ``mix`` fp32 [streams,
+    streams] indexed [from, to]). With ``nxt`` = (read [streams], weight, bias, alpha) the next sublayer's input is made
+    in the same pass from the new streams and returned in ``out_dtype``: tanh(alpha * sum_r read[r] * new[r]) * weight +
+    bias."""
+    _dev(x, y, mix, out_w)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous() or y.dtype != torch.float32 or y.dim() != 2 \
+            or y.stride(1) != 1 or y.shape[0] != x.shape[0] or x.shape[1] % y.shape[1]:
+        raise KernelError("streams_write takes contiguous fp32 streams [n, streams x width] and fp32 rows [n, width]")
+    n, width = y.shape
+    S = x.shape[1] // width
+    if not 1 <= S <= MAX_STREAMS:
+        raise KernelError(f"streams_write: {S} streams (1..{MAX_STREAMS} are taken)")
+    for t, k in ((mix, S * S), (out_w, S)):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != k:
+            raise KernelError(f"streams_write: the mixing matrix and the output weights are contiguous fp32 tensors of {S * S} and {S} entries")
+    out = None
+    read = w = b = alpha = None
+    if nxt is not None:
+        read, w, b, alpha = nxt
+        _dev(read, w, b, alpha)
+        _dyt(w, b, alpha, width)
+        if read.dtype != torch.float32 or not read.is_contiguous() or read.numel() != S:
+            raise KernelError(f"streams_write: the next read's weights are a contiguous fp32 tensor of {S} entries")
+        out = activation_rows(n, width, out_dtype or torch.float32, x.device)
+    _call("jllm_streams_write", _ptr(x), _ptr(y), y.stride(0), n, width, S, _ptr(mix), _ptr(out_w), _ptr(read), _ptr(w),
+          _ptr(b), _ptr(alpha), _ptr(out), _code(out.dtype) if out is not None else F32, out.stride(0) if out is not None else 0,
+          _stream())
     return out
 
 
@@ -1109,11 +1192,13 @@ def qkv_prepare(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torc
                 maps: int, dk: int, dv: int, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
                 gq: Optional[torch.Tensor] = None, gk: Optional[torch.Tensor] = None, eps: float = 0.0,
                 cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dims: int = 0,
-                temp_coef: float = 0.0, temp_every: int = 0) -> None:
+                temp_coef: float = 0.0, temp_every: int = 0, norm_per_head: bool = False,
+                pairing: str = "interleaved") -> None:
     """In place on the first columns of ``qkv`` rows [q: heads x maps x dk | k: kv_heads x maps x dk | v: kv_heads x
-    dv]: with ``gq``/``gk`` an RMS norm with those gains over the whole of q and the whole of k; with ``rot_dims`` the
-    rotation of the pairs (2i, 2i + 1) among the first ``rot_dims`` entries of every q and k head by the table rows of
-    the positions; with ``temp_every`` q times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1); then k and v go to
+    dv]: with ``gq``/``gk`` an RMS norm with those gains over the whole of q and the whole of k (``norm_per_head``: over
+    every head alone, with gains [dk] shared by the heads); with ``rot_dims`` the rotation of the pairs (2i, 2i + 1)
+    (``pairing`` "half": (i, i + rot_dims / 2)) among the first ``rot_dims`` entries of every q and k head by the table
+    rows of the positions; with ``temp_every`` q times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1); then k and v go to
     the rows' ``slots`` in the pages (``slots`` None or negative entries: nothing is stored)."""
     _dev(qkv, positions, slots, gq, gk, cos, sin, k_cache, v_cache)
     _rows2d(qkv, "qkv")
@@ -1126,26 +1211,38 @@ def qkv_prepare(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torc
     _tables(cos, sin, rot_dims)
     if (gq is None) != (gk is None):
         raise KernelError("the norm over the projections takes gains for both q and k")
-    if gq is not None and (gq.numel() != q_slots * dk or gk.numel() != k_slots * dk):
+    if pairing not in ("interleaved", "half"):
+        raise KernelError(f"qkv_prepare: pairing '{pairing}' ('interleaved' and 'half' are built)")
+    if gq is not None and norm_per_head and (gq.numel() != dk or gk.numel() != dk):
+        raise KernelError(f"the gains of the heads' norm must have {dk} entries each")
+    if gq is not None and not norm_per_head and (gq.numel() != q_slots * dk or gk.numel() != k_slots * dk):
         raise KernelError(f"the gains of the norm over the projections must have {q_slots * dk} and {k_slots * dk} entries")
     gd = _same_type("the gains of q and k", gq, gk)
     _check_kv_pages(k_cache, v_cache, k_slots, kv_heads, dk, dv, qkv.dtype)
     _call("jllm_qkv_prepare", _ptr(qkv), qkv.stride(0), _code(qkv.dtype), T, _ptr(positions), _ptr(slots), q_slots, k_slots,
           kv_heads, dk, dv, _ptr(gq), _ptr(gk), gd, float(eps), _ptr(cos), _ptr(sin), int(rot_dims), float(temp_coef),
-          int(temp_every), _ptr(k_cache), _ptr(v_cache), k_cache.shape[2], _stream())
+          int(temp_every), _ptr(k_cache), _ptr(v_cache), k_cache.shape[2], 1 if norm_per_head else 0,
+          1 if pairing == "half" else 0, _stream())
 
 
 def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                  row_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, maps: int, dk: int, dv: int,
                  scale: float, *, softcap: float = 0.0, window: int = 0, out_dtype: Optional[torch.dtype] = None,
-                 meta=None, exact: bool = False, defer_merge: bool = False):
+                 meta=None, exact: bool = False, defer_merge: bool = False, keep_first: int = 0,
+                 sinks: Optional[torch.Tensor] = None):
     """Causal attention of every row of ``q`` [T, heads x maps x dk] over its request's pages, keys [pages, kv_heads x
     maps, page_size, dk] and values [pages, kv_heads, page_size, dv]: map m of head h reads key slot (h / (heads /
     kv_heads)) * maps + m and value head h / (heads / kv_heads). Scores (q . k) * scale, capped as softcap * tanh(score
     / softcap) when ``softcap`` > 0. Returns [T, heads x maps x dv] in ``out_dtype`` (default: q's). With
     ``defer_merge`` a step whose rows were computed in key ranges comes back as a ``SplitHeads`` (the ranges' sums,
-    unmerged), which ``heads_finish`` takes in place of the tensor and merges in its prologue."""
-    _dev(q, k_cache, v_cache, block_table, row_req, positions)
+    unmerged), which ``heads_finish`` takes in place of the tensor and merges in its prologue. With ``window`` > 0 the
+    query at p sees keys p + 1 - window .. p and, with ``keep_first``, the keys before ``keep_first`` as well.
+    ``sinks`` (fp32 [heads], one map per head): exp(sink_h) joins head h's softmax denominator and has no value."""
+    _dev(q, k_cache, v_cache, block_table, row_req, positions, sinks)
+    if sinks is not None and (sinks.dtype != torch.float32 or not sinks.is_contiguous() or sinks.numel() != heads or maps != 1):
+        raise KernelError(f"attention: the sinks must be a contiguous fp32 tensor of {heads} entries (and one map per head)")
+    if keep_first < 0:
+        raise KernelError(f"attention: {keep_first} first keys kept")
     _rows2d(q, "q")
     T = q.shape[0]
     if q.shape[1] != heads * maps * dk:
@@ -1160,14 +1257,15 @@ def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
         return out
     if not exact and _fast_attention_dv is not None:
         got = _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, maps, dk, dv, scale,
-                                 softcap, window, meta, defer_merge)
+                                 softcap, window, meta, defer_merge, keep_first, sinks)
         if got is not False:
             return out if got is True else got
     if not exact:
         _count("general", "jllm_attention_dv_generic")
     _call("jllm_attention_dv_generic", _ptr(q), q.stride(0), _code(q.dtype), _ptr(out), out.stride(0), _code(out.dtype),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads,
-          kv_heads, maps, dk, dv, k_cache.shape[2], int(window), float(scale), float(softcap), _stream())
+          kv_heads, maps, dk, dv, k_cache.shape[2], int(window), float(scale), float(softcap), int(keep_first), _ptr(sinks),
+          _stream())
     return out
 
 
@@ -1178,12 +1276,13 @@ class SplitHeads:
     """Attention rows that were computed in key ranges and are not merged yet: ``partial`` fp32 [rows x (heads x maps) x
     splits x (dv + 2)] (a range's unnormalised sums, its maximum as an exponent of two, its sum)."""
 
-    def __init__(self, partial: torch.Tensor, splits: int, rows: int, slots: int, dv: int):
+    def __init__(self, partial: torch.Tensor, splits: int, rows: int, slots: int, dv: int, sinks=None):
         self.partial, self.splits, self.rows, self.slots, self.dv = partial, splits, rows, slots, dv
+        self.sinks = sinks  # fp32 [heads] or None: joins the denominator when the ranges are merged
 
 
 def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, maps, dk, dv, scale,
-                       softcap, window, meta, defer_merge=False):
+                       softcap, window, meta, defer_merge=False, keep_first=0, sinks=None):
     """The matrix-core kernel: bf16 pages, fp32 out, and the step's rows cut into tiles by the caller (``meta``:
     "tiles_dev" int32 [n_tiles, 4] as (request, first row, rows, first position or -1), "n_tiles")."""
     tiles = meta.get("tiles_dev") if meta else None
@@ -1210,9 +1309,9 @@ def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions
     ran = _try("jllm_attention_dv_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                _ptr(block_table), block_table.shape[1], _ptr(tiles), n_tiles, _ptr(positions), heads, kv_heads, maps, dk, dv,
                k_cache.shape[2], int(window), float(scale), float(softcap), splits, per_split, _ptr(partial),
-               T if meta.get("single_rows") else -1, 1 if defer else 0, _stream())
+               T if meta.get("single_rows") else -1, 1 if defer else 0, int(keep_first), _ptr(sinks), _stream())
     if ran and defer:
-        return SplitHeads(partial, splits, T, heads * maps, dv)
+        return SplitHeads(partial, splits, T, heads * maps, dv, sinks)
     return ran
 
 
@@ -1225,10 +1324,11 @@ HEAD_GATES = {"sigmoid": 0, "silu": 1}
 def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: torch.dtype, *, lam: float = 0.0,
                  normed: bool = False, eps: float = 0.0, norm_mul: float = 1.0, gain: Optional[torch.Tensor] = None,
                  gate: Optional[torch.Tensor] = None, gate_fn: str = "sigmoid", out: Optional[torch.Tensor] = None,
-                 out_mul: float = 1.0) -> torch.Tensor:
+                 out_mul: float = 1.0, gate_per_head: bool = False) -> torch.Tensor:
     """From a mixer's heads [T, heads x maps x dv] to the output product's input [T, heads x dv]: with two maps
     o = a1 - lam * a2; ``normed``: o / sqrt(mean(o^2) + eps) * norm_mul per head (times ``gain`` [dv]); with ``gate``
-    ([T, heads x dv], a view with any row stride) times sigmoid(gate) or, ``gate_fn`` "silu", silu(gate); times
+    ([T, heads x dv], a view with any row stride; ``gate_per_head``: [T, heads], one number for a whole head) times
+    sigmoid(gate) or, ``gate_fn`` "silu", silu(gate); times
     ``out_mul``. ``out``: where to write (a view with any row stride, [T, heads x dv]) instead of a new tensor."""
     if gate_fn not in HEAD_GATES:
         raise KernelError(f"heads_finish: gate function '{gate_fn}' ({sorted(HEAD_GATES)} are built)")
@@ -1246,8 +1346,8 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
             raise KernelError(f"attention rows have {att.shape[1]} entries, expected {heads * maps * dv}")
     if gate is not None:
         _rows2d(gate, "gate")
-        if gate.shape != (T, heads * dv):
-            raise KernelError(f"the gate is {tuple(gate.shape)}, expected {(T, heads * dv)}")
+        if gate.shape != (T, heads if gate_per_head else heads * dv):
+            raise KernelError(f"the gate is {tuple(gate.shape)}, expected {(T, heads if gate_per_head else heads * dv)}")
     if gain is not None and (gain.numel() != dv or not gain.is_contiguous()):
         raise KernelError(f"the heads' gain must have {dv} entries")
     if out is None:
@@ -1263,12 +1363,12 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
         _call("jllm_heads_finish_split", _ptr(att), split.splits, T, heads, maps, dv, float(lam), 1 if normed else 0, float(eps),
               float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
               gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, HEAD_GATES[gate_fn],
-              float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), _stream())
+              float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), 1 if gate_per_head else 0, _ptr(split.sinks), _stream())
         return out
     _call("jllm_heads_finish", _ptr(att), att.stride(0), _code(att.dtype), T, heads, maps, dv, float(lam), 1 if normed else 0,
           float(eps), float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
           gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, HEAD_GATES[gate_fn],
-          float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), _stream())
+          float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), 1 if gate_per_head else 0, _stream())
     return out
 
 
@@ -1451,11 +1551,15 @@ class MoeRouting:
         return self.tile_rows == MOE_TILE_ROWS_MANY
 
 
-def moe_router(z: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float):
-    """From the router's fp32 logits ``z`` [T, experts]: s = sigmoid(z); the choice scores are s + ``correction``; the
-    experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest choice scores and
-    only the ``keep`` best groups can be chosen from; the ``top`` largest choice scores among those win. Returns the
-    chosen experts (int32 [T, top]) and their weights (fp32 [T, top]): s of the chosen / (their sum + 1e-20) * scale."""
+def moe_router(z: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float,
+               score: str = "sigmoid", group_score: str = "top2", normalize: bool = True):
+    """From the router's fp32 logits ``z`` [T, experts]: s = sigmoid(z) (``score`` "softmax": softmax over all experts);
+    the choice scores are s + ``correction``; the experts form ``groups`` equal groups of neighbours, a group's score is
+    the sum of its two largest choice scores (``group_score`` "max": the largest) and only the ``keep`` best groups can be
+    chosen from; the ``top`` largest choice scores among those win. Returns the chosen experts (int32 [T, top]) and their
+    weights (fp32 [T, top]): s of the chosen / (their sum + 1e-20) * scale, or, not ``normalize``, s * scale."""
+    if score not in ("sigmoid", "softmax") or group_score not in ("top2", "max"):
+        raise KernelError(f"moe_router: score '{score}' (sigmoid, softmax) with group score '{group_score}' (top2, max)")
     _dev(z, correction)
     _rows2d(z, "router logits")
     if z.dtype != torch.float32:
@@ -1468,7 +1572,8 @@ def moe_router(z: torch.Tensor, correction: Optional[torch.Tensor], groups: int,
     if T == 0:
         return chosen, weights
     _call("jllm_moe_router", _ptr(z), z.stride(0), _ptr(correction), _code(correction.dtype) if correction is not None else F32,
-          T, E, int(groups), int(keep), int(top), float(scale), _ptr(chosen), _ptr(weights), _stream())
+          T, E, int(groups), int(keep), int(top), float(scale), _ptr(chosen), _ptr(weights), 1 if score == "softmax" else 0,
+          1 if group_score == "max" else 0, 1 if normalize else 0, _stream())
     return chosen, weights
 
 
@@ -1532,10 +1637,19 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, w2: Optio
 
 
 def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float, place_of: Optional[torch.Tensor] = None,
-                weights: Optional[torch.Tensor] = None) -> None:
+                weights: Optional[torch.Tensor] = None, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None, overwrite: bool = False) -> None:
     """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending); with ``place_of`` the k-th row of t is
-    y[place_of[t * top + k]]; with ``weights`` (fp32 [T, top]) the k-th term is also multiplied by weights[t, k]."""
-    _dev(y, residual, place_of, weights)
+    y[place_of[t * top + k]]; with ``weights`` (fp32 [T, top]) the k-th term is also multiplied by weights[t, k]. With
+    ``shared`` (fp32 [T, width], a shared expert's rows; it may be ``residual`` itself) its row t joins the sum, times
+    sigmoid(shared_gate[t]) where ``shared_gate`` (fp32 [T], any stride) is given; ``overwrite``: the rows of
+    ``residual`` are written instead of added to."""
+    _dev(y, residual, place_of, weights, shared, shared_gate)
+    if shared is not None and (shared.dtype != torch.float32 or not shared.is_contiguous() or shared.shape != residual.shape):
+        raise KernelError("moe_combine: the shared rows must be a contiguous fp32 tensor of the residual's shape")
+    if shared_gate is not None and (shared is None or shared_gate.dtype != torch.float32 or shared_gate.dim() != 1
+                                    or shared_gate.shape[0] != residual.shape[0]):
+        raise KernelError("moe_combine: the shared rows' gate is one fp32 number per row, beside the shared rows")
     T, width = residual.shape
     if y.dtype != torch.float32 or residual.dtype != torch.float32 or not y.is_contiguous() or not residual.is_contiguous() \
             or y.shape != (T * top, width):
@@ -1543,7 +1657,8 @@ def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float
     _i32(place_of, T * top, "places")
     if weights is not None and (weights.dtype != torch.float32 or not weights.is_contiguous() or weights.numel() != T * top):
         raise KernelError("moe_combine: the weights must be a contiguous fp32 [T, top] tensor")
-    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _ptr(weights), _stream())
+    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _ptr(weights),
+          _ptr(shared), _ptr(shared_gate), shared_gate.stride(0) if shared_gate is not None else 0, 1 if overwrite else 0, _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

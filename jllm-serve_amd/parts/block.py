@@ -14,6 +14,8 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import ops
+from ..weights.loader import WeightSpec
 from .base import Part, part_factory, register_part
 
 
@@ -217,3 +219,107 @@ class ParallelBlock(Part):
 
 
 register_part("arrangement", "parallel", ParallelBlock, replace=True)
+
+
+class StreamReader:
+    """How a sublayer of a hyper-connected layer gets its input: the weighted sum of the row's streams, then the norm.
+    The block before may have made it already, in the launch that wrote the streams (``HyperBlock.forward(next_norm=)``)."""
+
+    def __init__(self, read_name: str, norm):
+        self.read_name = read_name
+        self.norm = norm
+        self.read = None  # fp32 [streams]
+
+    def vectors(self):
+        return (self.read,) + tuple(self.norm.vectors())
+
+    def forward(self, x):
+        return self.norm.forward(x, read=self.read)
+
+
+class HyperBlock(Part):
+    """Hyper-connections: a row has ``streams`` copies x_1 .. x_s of the residual (fp32, side by side). Sublayer q (the
+    mixer, then the feed-forward) reads u = sum_s in_q[s] x_s, computes y = sublayer(norm_q(u)), and all streams are
+    rewritten at once from the old ones: x_t <- sum_s mix_q[s, t] x_s + out_q[t] * y. The weights are the tensors
+    ``<prefix>.<name>.in`` [streams], ``.out`` [streams] and ``.mix`` [streams, streams] (indexed [from, to]), held in
+    fp32. Writing the streams and reading the next sublayer's input from them is one launch (``ops.streams_write``), so
+    a layer costs two such launches beside its sublayers; the norm must be one that takes no statistics of the row
+    (``vectors()``: Dynamic Tanh)."""
+
+    chains_norms = True
+
+    def __init__(self, spec, prefix, build, positions):
+        ending = getattr(spec, "name_ending", ".weight")
+        self.streams = int(spec.streams)
+        if not 1 <= self.streams <= ops.MAX_STREAMS:
+            raise ValueError(f"{prefix}: {self.streams} residual streams (1..{ops.MAX_STREAMS} are built)")
+        self.width = build.hidden
+        self.dtype = build.dtype
+        make = part_factory("norm", spec.norm.kind)
+        norm1 = make(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}{ending}", build)
+        if not hasattr(norm1, "vectors"):
+            raise ValueError(f"{prefix}: the hyper arrangement reads its streams inside the norm's launch; norm '{spec.norm.kind}' does not offer that")
+        self.names = [f"{prefix}.{n}" for n in spec.hyper_names]
+        self.norm_in = StreamReader(self.names[0] + ".in", norm1)
+        mixer_prefix = f"{prefix}.{spec.mixer_prefix}" if getattr(spec, "mixer_prefix", "") else prefix
+        self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, mixer_prefix, build, positions)
+        if spec.ffn is None:
+            self.norm_post = self.ffn = None
+            self.parts = (norm1, self.mixer)
+        else:
+            norm2 = make(spec.norm, build.hidden, f"{prefix}.{spec.norm_post_name}{ending}", build)
+            self.norm_post = StreamReader(self.names[1] + ".in", norm2)
+            self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
+            self.parts = (norm1, self.mixer, norm2, self.ffn)
+        self.capturable = all(getattr(p, "capturable", True) for p in self.parts)
+        self.mix = [None, None]
+        self.out = [None, None]
+
+    def _sublayers(self):
+        return 1 if self.ffn is None else 2
+
+    def weight_specs(self):
+        s = self.streams
+        out = [w for p in self.parts for w in p.weight_specs()]
+        for n in self.names[:self._sublayers()]:
+            out += [WeightSpec(n + ".in", (s,), init="gain"), WeightSpec(n + ".out", (s,), init="gain"),
+                    WeightSpec(n + ".mix", (s, s), init="matrix")]
+        return out
+
+    def load(self, get):
+        for p in self.parts:
+            p.load(get)
+        readers = (self.norm_in, self.norm_post)
+        for q in range(self._sublayers()):
+            readers[q].read = get(self.names[q] + ".in").float().contiguous()
+            self.out[q] = get(self.names[q] + ".out").float().contiguous()
+            self.mix[q] = get(self.names[q] + ".mix").float().contiguous()
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def state_spec(self):
+        return self.mixer.state_spec()
+
+    def step_planners(self):
+        return [pl for p in self.parts for pl in (p.step_planners() if hasattr(p, "step_planners") else [])]
+
+    def _write(self, q, x, y, then):
+        """The streams' update behind sublayer q; returns ``then``'s input from the new streams (or None)."""
+        nxt = then.vectors() if isinstance(then, StreamReader) else None
+        return ops.streams_write(x, y, self.mix[q], self.out[q], nxt=nxt, out_dtype=self.dtype)
+
+    def forward(self, x, step, slot, normed_in=None, next_norm=None):
+        """``x``: fp32 [rows, streams x width]. ``normed_in``: this block's first input as the block before left it (a
+        tensor) or None; ``next_norm``: the ``StreamReader`` of the block that runs next. Returns its input when the
+        last write made it."""
+        xb = normed_in if isinstance(normed_in, torch.Tensor) else self.norm_in.forward(x)
+        y = sublayer_output(self.mixer, xb, step, slot, self.width)
+        if self.ffn is None:
+            return self._write(0, x, y, next_norm)
+        xb = self._write(0, x, y, self.norm_post)
+        y = sublayer_output(self.ffn, xb, step, None, self.width)
+        return self._write(1, x, y, next_norm)
+
+
+register_part("arrangement", "hyper", HyperBlock, replace=True)

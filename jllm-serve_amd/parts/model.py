@@ -36,6 +36,16 @@ class DecoderModel:
                        for l in config.layers]
         self.final_norm = part_factory("norm", config.final_norm.kind)(config.final_norm, config.hidden,
                                                                       config.names.final_norm, self.build)
+        # a norm over the embedding output, and several residual streams per row (all start as the embedding output;
+        # the final norm reads their sum): both need a norm part whose forward takes ``read`` / ``copies``
+        self.streams = int(getattr(config, "streams", 1))
+        self.embed_norm = None
+        if getattr(config, "embed_norm", None) is not None:
+            self.embed_norm = part_factory("norm", config.embed_norm.kind)(config.embed_norm, config.hidden,
+                                                                          config.names.embed_norm, self.build)
+        if self.streams > 1 and (self.embed_norm is None or not hasattr(self.final_norm, "vectors")):
+            raise ValueError("several residual streams need an embedding norm that writes them and a final norm that reads their sum")
+        self.streams_sum = None
         self.embed = None
         self.lm_head = None
         # vectors that join the stream before a run (config: ScheduleEntry.add_before), by tensor name
@@ -61,6 +71,8 @@ class DecoderModel:
             specs += p.weight_specs() if hasattr(p, "weight_specs") else []
         specs += [WeightSpec(name, (rows, c.hidden), init="bias") for name, rows in self.stream_vector_rows.items()]
         specs += [WeightSpec(name, (c.hidden, 2 * c.hidden)) for name in self.stream_mix_names]
+        if self.embed_norm is not None:
+            specs += self.embed_norm.weight_specs()
         for l in self.layers:
             specs += l.weight_specs()
         specs += self.final_norm.weight_specs()
@@ -80,6 +92,10 @@ class DecoderModel:
                 p.load(get)
         self.stream_vectors = {name: get(name) for name in self.stream_vector_rows}
         self.stream_mixes = {name: get(name) for name in self.stream_mix_names}
+        if self.embed_norm is not None:
+            self.embed_norm.load(get)
+        if self.streams > 1:
+            self.streams_sum = torch.ones(self.streams, dtype=torch.float32, device=self.device)
         for l in self.layers:
             l.load(get)
         self.final_norm.load(get)
@@ -114,6 +130,9 @@ class DecoderModel:
         for p in self.positions:  # an encoding that is added to the embedded rows rather than applied in the mixers
             if hasattr(p, "embed_add"):
                 p.embed_add(x, step)
+        if self.embed_norm is not None:  # the stream stays fp32; with several streams every one starts as this row
+            x = self.embed_norm.forward(x, out_dtype=torch.float32, copies=self.streams) if hasattr(self.embed_norm, "vectors") \
+                else self.embed_norm.forward(x).float()
         schedule = self.config.schedule
         x0 = x.clone() if self.stream_mix_names else None  # the embedding output, for the runs that mix it back in
         carry = None  # the next block's input norm, when the block before prepared it (parts/block.py)
@@ -147,9 +166,10 @@ class DecoderModel:
                     if nxt_e is not None and (nxt_e.add_before is not None or nxt_e.mix_before is not None):
                         next_norm = None  # the stream changes before the next block reads it
                     carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm)
-            if self.watch is not None:
-                self.watch(run, x)
+            if self.watch is not None:  # (with several streams: their sum)
+                self.watch(run, x if self.streams == 1 else x.view(x.shape[0], self.streams, -1).sum(dim=1))
         if step.n_selected == 0:
             return torch.empty((0, self.config.vocab), dtype=torch.float32, device=self.device)
-        xs = self.final_norm.forward(x, rows=step.selected)
+        xs = self.final_norm.forward(x, rows=step.selected) if self.streams == 1 else \
+            self.final_norm.forward(x, rows=step.selected, read=self.streams_sum)
         return ops.gemm(xs, self.lm_head, out_dtype=torch.float32, exact=self.build.exact)

@@ -1,10 +1,11 @@
-"""RMSNorm: y = (x * rsqrt(mean(x^2) + eps)) * g over fp32 rows (cpu/VectorKernels.java:630-634), and layer norm with a
-weight and a bias: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b."""
+"""RMSNorm: y = (x * rsqrt(mean(x^2) + eps)) * g over fp32 rows (cpu/VectorKernels.java:630-634), layer norm with a
+weight and a bias: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b, and Dynamic Tanh, which takes no statistics
+of the row: y = tanh(alpha x) w + b."""
 from __future__ import annotations
 
 import torch
 
-from ..config.schema import LayerNormSpec, NormSpec
+from ..config.schema import DynTanhSpec, LayerNormSpec, NormSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import BuildContext, Part, register_part
@@ -108,3 +109,38 @@ class LayerNorm(Part):
 
 
 register_part("norm", "layernorm", LayerNorm, replace=True)
+
+
+class DynTanh(Part):
+    """tanh(alpha * x) * w + b element by element in fp32 (weight, bias and slope are held in fp32 whatever the run's
+    type): no mean, no variance, no eps. ``forward`` also reads several residual streams as one weighted sum first
+    (``read`` fp32 [streams], ``x`` [rows, streams x width]) and can write its result several times side by side."""
+
+    def __init__(self, spec: DynTanhSpec, dim: int, weight_name: str, build: BuildContext):
+        self.dim = dim
+        self.weight_name = weight_name
+        self.bias_name = weight_name + spec.bias_suffix
+        self.alpha_name = weight_name + spec.alpha_suffix
+        self.out_dtype = build.dtype
+        self.gain = self.bias = self.alpha = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.weight_name, (self.dim,), init="gain"), WeightSpec(self.bias_name, (self.dim,), init="bias"),
+                WeightSpec(self.alpha_name, (), init="gain")]
+
+    def load(self, get):
+        self.gain = get(self.weight_name).float().contiguous()
+        self.bias = get(self.bias_name).float().contiguous()
+        self.alpha = get(self.alpha_name).float().reshape(1).contiguous()
+
+    def vectors(self):
+        """(weight, bias, alpha) as the stream kernels take them."""
+        return self.gain, self.bias, self.alpha
+
+    def forward(self, x, rows=None, read=None, out_dtype=None, copies=1):
+        streams = read.numel() if read is not None else 1
+        return ops.dyntanh(x, self.gain, self.bias, self.alpha, out_dtype or self.out_dtype, streams=streams, read=read,
+                           rows=rows, copies=copies)
+
+
+register_part("norm", "dyntanh", DynTanh, replace=True)

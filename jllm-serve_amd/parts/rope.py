@@ -13,7 +13,9 @@ import math
 import numpy as np
 import torch
 
-from ..config.schema import RopeScaling, RopeSpec
+from ..config.schema import LearnedPositionSpec, RopeScaling, RopeSpec
+from ..kernels import ops
+from ..weights.loader import WeightSpec
 from .base import BuildContext, Part, register_part
 
 
@@ -89,3 +91,31 @@ class RotaryPosition(Part):
 
 
 register_part("position", "rope", RotaryPosition, replace=True)
+
+
+class LearnedPosition(Part):
+    """A learned vector per position, added to the embedded rows once at the input (the model calls ``embed_add``); the
+    mixers rotate nothing by it."""
+
+    def __init__(self, spec: LearnedPositionSpec, build: BuildContext):
+        self.spec = spec
+        self.width = build.hidden
+        self.table = None
+
+    def rotary(self):
+        return None
+
+    def weight_specs(self):
+        return [WeightSpec(self.spec.name, (self.spec.rows, self.width))]
+
+    def load(self, get):
+        self.table = get(self.spec.name)
+
+    def embed_add(self, x, step):
+        last = max((s.pos0 + s.n for s in step.segments), default=0)  # (a captured step has no host-side segments)
+        if last > self.spec.rows:
+            raise ValueError(f"a request reaches position {last - 1}, the position table has {self.spec.rows} rows")
+        ops.gather_add(x, self.table, step.positions)
+
+
+register_part("position", "learned_position", LearnedPosition, replace=True)

@@ -1,7 +1,9 @@
 """Causal grouped-query attention over the paged cache with key and value sizes of their own, and what several designs
 put around the softmax (config/schema.py: WideAttentionSpec): two score maps per head whose outputs are subtracted
-(differential attention), a norm with gains over the whole q and k projections, rotation of neighbouring pairs, capped
-scores, a query scale that grows with the position, an output gate.
+(differential attention), a norm with gains over the whole q and k projections or over every head alone, rotation of
+neighbouring pairs or of the two halves of a head's rotated part, capped scores, a query scale that grows with the
+position, a sliding window that may keep the first keys, a learned sink in the softmax's denominator, an output gate per
+channel or per head.
 
 A step is
   1. one product with the stacked weight [W_q | W_k | W_v | W_g] and the stacked bias (zeros for the gate's rows),
@@ -48,15 +50,18 @@ class WideAttention(Part):
     def __init__(self, spec: WideAttentionSpec, prefix: str, build: BuildContext, positions):
         if spec.maps not in (1, 2):
             raise ValueError(f"{prefix}: {spec.maps} score maps per head (one or two are built)")
-        if spec.qk_norm not in (None, "whole"):
-            raise ValueError(f"{prefix}: q/k norm '{spec.qk_norm}' is not built for this mixer ('whole' is)")
+        if spec.qk_norm not in (None, "whole", "head"):
+            raise ValueError(f"{prefix}: q/k norm '{spec.qk_norm}' is not built for this mixer ('whole' and 'head' are)")
+        if spec.sink and spec.maps != 1:
+            raise ValueError(f"{prefix}: a sink with {spec.maps} score maps per head")
+        if spec.keep_first and not spec.window:
+            raise ValueError(f"{prefix}: first keys are kept beside a window, and this mixer has none")
         self.spec = spec
         self.prefix = prefix
         self.build = build
         self.position = positions[spec.position] if spec.position is not None else None
         rot = self.position.rotary() if self.position is not None else None
-        if rot is not None and getattr(self.position, "pairing", "half") != "interleaved":
-            raise ValueError(f"{prefix}: this mixer's kernels rotate the pairs (2i, 2i + 1) only")
+        self.pairing = getattr(self.position, "pairing", "half") if rot is not None else "interleaved"
         self.rot = rot
         try:
             ops.check_attention_dv_shape(spec.heads, spec.kv_heads, spec.maps, spec.dim, spec.vdim, rot[2] if rot else 0)
@@ -66,6 +71,8 @@ class WideAttention(Part):
         self.k_dim = spec.kv_heads * spec.maps * spec.dim
         self.v_dim = spec.kv_heads * spec.vdim
         self.o_dim = spec.heads * spec.vdim
+        self.gate_dim = spec.heads if spec.gate_per_head else self.o_dim  # rows of W_g: one per head, or one per channel
+        self.sinks = None
         self.w_in = self.b_in = self.w_o = self.g_q = self.g_k = None
         self.lam = 0.0
 
@@ -82,10 +89,15 @@ class WideAttention(Part):
         if s.qk_norm == "whole":
             out += [WeightSpec(self._name("q", nm.norm_suffix), (self.q_dim,), init="gain"),
                     WeightSpec(self._name("k", nm.norm_suffix), (self.k_dim,), init="gain")]
+        if s.qk_norm == "head":  # one gain vector for all q heads, one for all k heads
+            out += [WeightSpec(self._name("q", nm.norm_suffix), (s.dim,), init="gain"),
+                    WeightSpec(self._name("k", nm.norm_suffix), (s.dim,), init="gain")]
+        if s.sink:
+            out.append(WeightSpec(self._name("sink"), (s.heads,), init="bias"))
         if s.maps == 2:
             out += [WeightSpec(f"{self.prefix}.{n}", (s.dim,), init="bias") for n in nm.lambda_q + nm.lambda_k]
         if s.out_gate:
-            out.append(WeightSpec(self._name("gate"), (self.o_dim, d)))
+            out.append(WeightSpec(self._name("gate"), (self.gate_dim, d)))
         out.append(WeightSpec(self._name("o"), (d, self.o_dim)))
         return out
 
@@ -100,9 +112,11 @@ class WideAttention(Part):
         if s.bias:
             b = [get(self._name(n, nm.bias_suffix)).to(torch.float32) for n in "qkv"]
             if s.out_gate:
-                b.append(torch.zeros(self.o_dim, dtype=torch.float32, device=b[0].device))
+                b.append(torch.zeros(self.gate_dim, dtype=torch.float32, device=b[0].device))
             self.b_in = pad_rows(torch.cat(b).contiguous())
-        if s.qk_norm == "whole":
+        if s.sink:
+            self.sinks = get(self._name("sink")).float().contiguous()
+        if s.qk_norm in ("whole", "head"):
             self.g_q, self.g_k = get(self._name("q", nm.norm_suffix)), get(self._name("k", nm.norm_suffix))
             if self.g_q.dtype != self.g_k.dtype:
                 self.g_q, self.g_k = self.g_q.float(), self.g_k.float()
@@ -114,7 +128,8 @@ class WideAttention(Part):
 
     def cache_spec(self):
         s = self.spec
-        return PageSpec((CacheRow("k", (s.kv_heads * s.maps, s.dim), 1), CacheRow("v", (s.kv_heads, s.vdim), 1)), s.window)
+        return PageSpec((CacheRow("k", (s.kv_heads * s.maps, s.dim), 1), CacheRow("v", (s.kv_heads, s.vdim), 1)), s.window,
+                        s.keep_first if s.window else 0)
 
     def step_planners(self):
         return [WideStepPlanner()]
@@ -155,15 +170,18 @@ class WideAttention(Part):
         cos, sin, rdims = self.rot if self.rot is not None else (None, None, 0)
         ops.qkv_prepare(y, step.positions, g.slots if slot.writes else None, s.heads, s.kv_heads, s.maps, s.dim, s.vdim,
                         k_cache, v_cache, gq=self.g_q, gk=self.g_k, eps=s.eps, cos=cos, sin=sin, rot_dims=rdims,
-                        temp_coef=s.q_temp_coef, temp_every=s.q_temp_every)
+                        temp_coef=s.q_temp_coef, temp_every=s.q_temp_every, norm_per_head=s.qk_norm == "head",
+                        pairing=self.pairing)
         meta = self._batch_facts(step)
         att = ops.attention_dv(y[:, :self.q_dim], k_cache, v_cache, g.block_table, step.row_req, step.positions, s.heads,
                                s.kv_heads, s.maps, s.dim, s.vdim, s.scale, softcap=s.softcap, window=s.window,
-                               out_dtype=torch.float32, meta=meta, exact=exact, defer_merge=True)
+                               out_dtype=torch.float32, meta=meta, exact=exact, defer_merge=True, keep_first=s.keep_first,
+                               sinks=self.sinks)
         gate_at = self.q_dim + self.k_dim + self.v_dim
-        gate = y[:, gate_at:gate_at + self.o_dim] if s.out_gate else None
+        gate = y[:, gate_at:gate_at + self.gate_dim] if s.out_gate else None
         return ops.heads_finish(att, s.heads, s.maps, s.vdim, self.build.dtype, lam=self.lam, normed=s.maps == 2,
-                                eps=s.eps, norm_mul=1.0 - s.diff, gate=gate, out=out, out_mul=out_mul)
+                                eps=s.eps, norm_mul=1.0 - s.diff, gate=gate, out=out, out_mul=out_mul,
+                                gate_per_head=bool(s.out_gate and s.gate_per_head))
 
     def output(self, xb, step, slot):
         """The mixer's output as fp32 rows of its own (for arrangements that norm or weigh it before the add)."""
