@@ -133,7 +133,9 @@ def parse_pivipel(c: Mapping[str, Any], model_type: str, architecture: str) -> M
     norm = DynTanhSpec()
     positions: List[Any] = [LearnedPositionSpec(name="pos", rows=longest)]
     layers: List[LayerSpec] = []
-    index_of = {}  # config layer -> index among the layers that have tensors
+    # config layer -> index among the layers that have tensors of their own
+    index_of = {i: n for n, i in enumerate(i for i, l in enumerate(raw_layers)
+                                           if isinstance(l, Mapping) and l.get("weights_of") is None)}
     schedule = []
     for i, layer in enumerate(raw_layers):
         where = f"layers[{i}]"
@@ -144,13 +146,14 @@ def parse_pivipel(c: Mapping[str, Any], model_type: str, architecture: str) -> M
         if owner is not None:
             j = _int(layer, "weights_of", where, least=0)
             if j not in index_of:
-                raise ConfigError(f"config.json: {where}.weights_of={j} names no earlier layer with tensors of its own")
+                raise ConfigError(f"config.json: {where}.weights_of={j} names no layer with tensors of its own")
+            if raw_layers[j].get("type") != kind:
+                raise ConfigError(f"config.json: {where} is '{kind}' and borrows the weights of a '{raw_layers[j].get('type')}' layer")
             schedule.append(ScheduleEntry(index_of[j]))  # the same weights, a cache of this run's own
             continue
         mixer = _mixer(kind, _need(layer, "mixer", where), where + ".mixer", eps, positions)
         mlp = layer.get("mlp")
         ffn = _ffn(mlp, where + ".mlp") if mlp is not None else None
-        index_of[i] = len(layers)
         schedule.append(ScheduleEntry(len(layers)))
         layers.append(LayerSpec(mixer=mixer, ffn=ffn, norm=norm, prefix=f"l{i}", arrangement="hyper" if hyper else "prenorm",
                                 norm_in_name="norm1", norm_post_name="norm2", name_ending="", mixer_prefix="mix",

@@ -15,7 +15,7 @@
 #include "common.h"
 
 #define ST_THREADS 256
-#define ST_MAX_STREAMS 8
+#define ST_MAX_STREAMS 16
 
 template <typename T>
 __global__ __launch_bounds__(ST_THREADS) void gather_add_kernel(float* __restrict__ x, int ldx, const T* __restrict__ table,

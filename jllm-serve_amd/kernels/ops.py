@@ -251,7 +251,7 @@ def gather_add(x: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
     _call("jllm_gather_add", _ptr(x), x.stride(0), _ptr(table), _code(table.dtype), table.shape[0], _ptr(ids), n, x.shape[1], _stream())
 
 
-MAX_STREAMS = 8   # residual streams per row that the stream kernels take (csrc/streams.hip)
+MAX_STREAMS = 16  # residual streams per row that the stream kernels take (csrc/streams.hip)
 
 
 def _dyt(weight, bias, alpha, width):

@@ -283,7 +283,11 @@ class HyperBlock(Part):
         out = [w for p in self.parts for w in p.weight_specs()]
         for n in self.names[:self._sublayers()]:
             out += [WeightSpec(n + ".in", (s,), init="gain"), WeightSpec(n + ".out", (s,), init="gain"),
-                    WeightSpec(n + ".mix", (s, s), init="matrix")]
+                    WeightSpec(n + ".mix", (s, s), init="eye")]
+        if self.ffn is None:  # a checkpoint may still carry the second sublayer's (unused) stream weights
+            n = self.names[1]
+            out += [WeightSpec(n + ".in", (s,), optional=True), WeightSpec(n + ".out", (s,), optional=True),
+                    WeightSpec(n + ".mix", (s, s), optional=True)]
         return out
 
     def load(self, get):

@@ -40,7 +40,8 @@ class WeightError(ValueError):
 @dataclass(frozen=True)
 class WeightSpec:
     """One tensor a part needs. ``init`` tells the random-weights mode how to fill it:
-    "matrix" N(0, std), "gain" 1 + N(0, gain_std), "bias" N(0, std), "zeros", "expert_table" (int32 [rows, top]:
+    "matrix" N(0, std), "gain" 1 + N(0, gain_std), "bias" N(0, std), "zeros", "eye" (a square matrix: the identity +
+    N(0, std)), "expert_table" (int32 [rows, top]:
     every row holds ``top`` different expert numbers below the count that the tensor's name is registered with). A
     dimension of -1 is the checkpoint's to choose (a narrow middle between two projections whose size no config key
     gives): any size matches, the part that declared it checks that its tensors agree, and the random-weights mode
@@ -162,4 +163,6 @@ class RandomSource:
             t = torch.randn(s.shape, generator=g, dtype=torch.float32, device=self.device) * self.gain_std + 1.0
         else:
             t = torch.randn(s.shape, generator=g, dtype=torch.float32, device=self.device) * self.std
+            if s.init == "eye":
+                t = t + torch.eye(s.shape[0], s.shape[1], dtype=torch.float32, device=self.device)
         return t.to(self._dtype)
