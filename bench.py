@@ -22,6 +22,9 @@ differential attention layers) beside the Qwen3 dense model of the same width, h
 `--workload compare --design ratasun [--size 2k|4k]` measures a Ratasun model (latent attention, a delta rule with a decay
 per key channel and a state-space layer, every layer with router-chosen experts beside the mixer) beside the Miforax
 model of the same width, heads, latent and experts.
+`--workload compare --design pivipel [--size 2k|4k]` measures a Pivipel model (several residual streams, Dynamic-Tanh
+norms, windowed attention with a sink or with kept first keys, dense and router-chosen expert layers in turn) beside the
+Miforax model of the same width, heads, window and feed-forwards.
 `--workload compare [--size 2k|4k]` is another run altogether: a Miforax model (latent attention with a window, dense
 and table-routed expert layers in turn) beside the closest model the engine had before, a Qwen3 dense model with the
 same width, layers, heads, window and feed-forward width, both with random weights: prefill of 2,048 tokens and
@@ -318,6 +321,95 @@ def compare_ratasun(args) -> dict:
     return out
 
 
+PIVIPEL_EXTRA = {  # what a Pivipel model has beyond the sizes it shares with the Miforax model of the same name
+    "2k": dict(streams=4, keep_first=64, groups=4, keep=2, rot_dims=64),
+    "4k": dict(streams=4, keep_first=64, groups=8, keep=4, rot_dims=64),
+}
+
+
+def pivipel_config(z: dict) -> dict:
+    """Layers of windowed attention, the rotated one with a sink and the one with q/k norms and kept first keys in turn;
+    dense and expert feed-forwards in turn as in the Miforax model of the same sizes (top x expert_ff + shared_ff = ff)."""
+    common = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": z["dim"] ** -0.5}
+    att = dict(common, mask={"size": z["window"]},
+               rot={"base": 1e6, "dims": z["rot_dims"], "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 4096}})
+    att2 = dict(common, mask={"size": z["window"], "keep_first": z["keep_first"]})
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"], "scale": 1.0, "groups": {"count": z["groups"], "keep": z["keep"]}},
+           "expert": {"ff": z["expert_ff"], "limit": 7.0}, "shared": {"ff": z["shared_ff"], "limit": 7.0}}
+    return {"architecture": "Pivipel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "max_positions": 8192,
+            "streams": z["streams"],
+            "layers": [{"type": "attention_2" if i % 2 else "attention", "mixer": att2 if i % 2 else att,
+                        "mlp": moe if i % 2 else dense} for i in range(z["layers"])]}
+
+
+class PivipelWork:
+    """Bytes and flops of passes over a Pivipel model of the sizes ``z`` (the interface of ``Work``). A decode step reads
+    every weight outside the experts, of the experts at most batch x top per layer, and per request the keys and values
+    its windows hold (and the kept first keys); a row costs 2 flops per weight it passes through (of the experts: top), and
+    per (row, key) pair and head 2 dim for the score and 2 vdim for the weighted sum. The streams (fp32, read and
+    written twice a layer) are activations and not counted."""
+
+    def __init__(self, z: dict, dtype: str):
+        self.z = z
+        self.L, self.d, self.H, self.Hkv, self.F, self.V, self.hd = z["layers"], z["width"], z["heads"], z["kv_heads"], z["ff"], z["vocab"], z["dim"]
+        self.window = z["window"]
+        self.esize = 2 if dtype == "bf16" else 4
+        self.dtype = dtype
+        d, H, G, dk, dv = self.d, self.H, self.Hkv, z["dim"], z["vdim"]
+        self.n_moe = self.L // 2
+        self.n_dense = self.L - self.n_moe
+        base = (H * dk + G * (dk + dv)) * d + d * H * dv
+        self.mixers = self.n_dense * (base + H * d) + self.n_moe * (base + H * dv * d)  # a gate per head / per channel
+        self.dense_ff = 3 * d * z["ff"]
+        self.shared_ff = 3 * d * z["shared_ff"] + (z["experts"] + 1) * d
+        self.expert = 3 * d * z["expert_ff"]
+        self.kv_bytes_per_token = self.L * G * (dk + dv) * self.esize
+        self.weight_bytes = (self.mixers + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + z["experts"] * self.expert)
+                             + self.V * d + 8192 * d) * self.esize
+
+    def decode_bytes(self, tokens_held: float, batch: int = 0) -> float:
+        z = self.z
+        touched = min(z["experts"], max(batch, 1) * z["top"])
+        w = self.mixers + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + touched * self.expert) + self.V * self.d
+        if batch:
+            tokens_held = min(tokens_held, float(self.window + z["keep_first"] / 2.0) * batch)
+        return w * self.esize + self.kv_bytes_per_token * tokens_held
+
+    def pairs(self, T: int) -> float:
+        return sum(min(i + 1, self.window) for i in range(T))
+
+    def flops(self, rows: float, pairs: float, selected: float) -> float:
+        per_row = self.mixers + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + self.z["top"] * self.expert)
+        return 2.0 * rows * per_row + 2.0 * self.H * (self.z["dim"] + self.z["vdim"]) * self.L * pairs + 2.0 * self.V * self.d * selected
+
+
+def compare_pivipel(args) -> dict:
+    """``--workload compare --design pivipel``: the Pivipel model of ``--size`` and the Miforax model of the same width,
+    heads, window and feed-forwards, one after the other: prefill of 2,048 tokens in one portion, decoding at batch 8 and
+    64 with every window full."""
+    z = dict(COMPARE_SIZES[args.size], **PIVIPEL_EXTRA[args.size])
+    ctx = z["window"] + 1024
+    decodes = [dict(key=f"b{B}", batch=B, prompt_len=z["window"] + 128, steps=args.point_steps, warmup=4) for B in (8, 64)]
+    prefills = [dict(key="main", tokens=2048, portion=2048)]
+    out = {"metric": f"Pivipel beside Miforax at equal sizes ({args.size})", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "higher_is_better": True,
+           "config": {"size": args.size, **z, "context": ctx, "page_size": PAGE}, "models": {}}
+    for name, shape, work in (("pivipel", pivipel_config(z), PivipelWork(z, "bf16")),
+                              ("miforax", miforax_config(z), LatentWork(z, "bf16"))):
+        r = steady(args, name, "bf16", 0, ctx, decodes, prefills, shape=shape, work=work)
+        m = {"prefill_2048_tok_s": r["prefill"]["main"]["value"], "prefill_2048_ms": r["prefill"]["main"]["ms"],
+             "prefill_flop_frac": r["prefill"]["main"]["frac"]}
+        for B in (8, 64):
+            s_, held, by = r["decode"][f"b{B}"]
+            m[f"decode_b{B}_tok_s"] = round(B / s_, 1)
+            m[f"decode_b{B}_ms"] = round(s_ * 1e3, 3)
+            m[f"decode_b{B}_hbm_frac"] = round(by / s_ / HBM_PEAK, 4)
+        out["models"][name] = m
+    out["value"] = out["models"]["pivipel"]["decode_b8_tok_s"]
+    return out
+
+
 def compare_kebepel(args) -> dict:
     """``--workload compare --design kebepel``: the Kebepel model of ``--size`` and the Qwen3 dense model of the same
     width, heads, head size and feed-forward, one after the other: prefill of 2,048 tokens in one portion, decoding at
@@ -492,9 +584,9 @@ def main() -> int:
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end; "
                          "compare: a Miforax model beside the Qwen3 dense model of the same sizes")
     ap.add_argument("--size", default="2k", choices=sorted(COMPARE_SIZES), help="compare: which sizes")
-    ap.add_argument("--design", default="miforax", choices=["miforax", "kebepel", "ratasun"],
-                    help="compare: which design stands beside the Qwen3 dense model of the same sizes (ratasun: beside the "
-                         "Miforax model of the same sizes)")
+    ap.add_argument("--design", default="miforax", choices=["miforax", "kebepel", "ratasun", "pivipel"],
+                    help="compare: which design stands beside the Qwen3 dense model of the same sizes (ratasun and pivipel: "
+                         "beside the Miforax model of the same sizes)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -504,7 +596,7 @@ def main() -> int:
         print(json.dumps(serve_workload(args)))
         return 0
     if args.workload == "compare":
-        run = {"kebepel": compare_kebepel, "ratasun": compare_ratasun}.get(args.design, compare_workload)
+        run = {"kebepel": compare_kebepel, "ratasun": compare_ratasun, "pivipel": compare_pivipel}.get(args.design, compare_workload)
         print(json.dumps(run(args)))
         return 0
 
