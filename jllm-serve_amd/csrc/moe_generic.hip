@@ -199,7 +199,8 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
                                                          int top, float weight, const int* __restrict__ place_of,
                                                          const float* __restrict__ weights, const float* __restrict__ shared,
-                                                         const float* __restrict__ shared_gate, int ldsg, int overwrite) {
+                                                         const float* __restrict__ shared_gate, int ldsg, int overwrite,
+                                                         int ld_shared) {
   const int t = blockIdx.x;
   // a shared expert's rows join the sum, times sigmoid of the row's gate logit where it has one
   const float sg = shared ? (shared_gate ? 1.0f / (1.0f + expf(-shared_gate[(size_t)t * ldsg])) : 1.0f) : 0.f;
@@ -210,20 +211,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
       s = weights ? fmaf(weights[(size_t)t * top + k], y[row * width + i], s) : s + y[row * width + i];
     }
     float r = overwrite ? 0.f : residual[(size_t)t * width + i];
-    if (shared) r = fmaf(sg, shared[(size_t)t * width + i], r);
+    if (shared) r = fmaf(sg, shared[(size_t)t * ld_shared + i], r);
     residual[(size_t)t * width + i] = r + weight * s;
   }
 }
 
-// `shared` [T, width] fp32 (optional): one more term per row, times sigmoid(shared_gate[t * ldsg]) where a gate is given;
+// `shared` [T, width] fp32, rows `ld_shared` apart (optional): one more term per row, times sigmoid(shared_gate[t * ldsg]) where a gate is given;
 // `overwrite`: the rows of `residual` are written, not added to (it may be the same tensor as `shared`)
 extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, const int* place_of,
                                 const float* weights, const float* shared, const float* shared_gate, int ldsg, int overwrite,
-                                hipStream_t stream) {
+                                int ld_shared, hipStream_t stream) {
   if (T <= 0) return 0;
   if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
   if (shared_gate && !shared) JLLM_FAIL("moe_combine: a gate without the shared rows it weighs");
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg, overwrite);
+  if (shared && ld_shared < width) JLLM_FAIL("moe_combine: shared rows %d apart for a width of %d", ld_shared, width);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg, overwrite,
+                                            ld_shared);
   JLLM_CHECK_LAUNCH("moe_combine");
   return 0;
 }

@@ -73,7 +73,7 @@ def _declare(lib) -> None:
         "jllm_latent_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
         "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
         "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
-        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P, _P, _P, _I, _I, _P],
+        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P, _P, _P, _I, _I, _I, _P],
         "jllm_moe_router": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _I, _I, _I, _P],
         "jllm_gather_add": [_P, _I, _P, _I, _I, _P, _I, _I, _P],
         "jllm_dyntanh_read": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P],
@@ -1641,12 +1641,12 @@ def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float
                 shared_gate: Optional[torch.Tensor] = None, overwrite: bool = False) -> None:
     """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending); with ``place_of`` the k-th row of t is
     y[place_of[t * top + k]]; with ``weights`` (fp32 [T, top]) the k-th term is also multiplied by weights[t, k]. With
-    ``shared`` (fp32 [T, width], a shared expert's rows; it may be ``residual`` itself) its row t joins the sum, times
+    ``shared`` (fp32 [T, width] with any row stride, a shared expert's rows) its row t joins the sum, times
     sigmoid(shared_gate[t]) where ``shared_gate`` (fp32 [T], any stride) is given; ``overwrite``: the rows of
     ``residual`` are written instead of added to."""
     _dev(y, residual, place_of, weights, shared, shared_gate)
-    if shared is not None and (shared.dtype != torch.float32 or not shared.is_contiguous() or shared.shape != residual.shape):
-        raise KernelError("moe_combine: the shared rows must be a contiguous fp32 tensor of the residual's shape")
+    if shared is not None and (shared.dtype != torch.float32 or shared.dim() != 2 or shared.stride(1) != 1 or shared.shape != residual.shape):
+        raise KernelError("moe_combine: the shared rows must be an fp32 tensor of the residual's shape with contiguous rows")
     if shared_gate is not None and (shared is None or shared_gate.dtype != torch.float32 or shared_gate.dim() != 1
                                     or shared_gate.shape[0] != residual.shape[0]):
         raise KernelError("moe_combine: the shared rows' gate is one fp32 number per row, beside the shared rows")
@@ -1658,7 +1658,8 @@ def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float
     if weights is not None and (weights.dtype != torch.float32 or not weights.is_contiguous() or weights.numel() != T * top):
         raise KernelError("moe_combine: the weights must be a contiguous fp32 [T, top] tensor")
     _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _ptr(weights),
-          _ptr(shared), _ptr(shared_gate), shared_gate.stride(0) if shared_gate is not None else 0, 1 if overwrite else 0, _stream())
+          _ptr(shared), _ptr(shared_gate), shared_gate.stride(0) if shared_gate is not None else 0, 1 if overwrite else 0,
+          shared.stride(0) if shared is not None else 0, _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:
