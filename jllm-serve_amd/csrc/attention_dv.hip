@@ -1,20 +1,26 @@
 // Causal attention over a paged cache whose keys and values have sizes of their own, with the options that several
 // designs put around the softmax: several score maps per head over shared values, a cap on the scores, a norm over a
-// whole projection, rotation of neighbouring pairs, a query scale that follows the position. fp32 or bf16 storage, all
-// arithmetic in fp32, any sizes. Three kernels:
+// whole projection or over every head, rotation of neighbouring pairs or of a head's halves, a query scale that follows
+// the position, a sliding window that may keep the first keys, a sink in the denominator, a gate per channel or per head.
+// fp32 or bf16 storage, all arithmetic in fp32, any sizes. Three kernels:
 //
 //   qkv_prepare      one workgroup per row of the stacked projection [q | k | v]: optional RMS norm with gains over the
-//                    whole of q and the whole of k; optional rotation of the pairs (2i, 2i + 1) among the first rot_dims
-//                    entries of every q and k head by the row's position; optional q *= 1 + coef * ln(floor((p + 1) /
-//                    every) + 1); q back in place, k and v into the row's place in the cache
+//                    whole of q and the whole of k (or over every head alone, with gains shared by the heads); optional
+//                    rotation of the pairs (2i, 2i + 1) (or (i, i + rot_dims / 2)) among the first rot_dims entries of
+//                    every q and k head by the row's position; optional q *= 1 + coef * ln(floor((p + 1) / every) + 1);
+//                    q back in place, k and v into the row's place in the cache
 //   attention_dv     one workgroup of four waves per (row, query slot). A query slot is one score map of one head: with
 //                    M maps per head and H heads over G key/value heads there are H * M query slots and G * M key slots;
 //                    query slot s reads key slot (s / (M * H / G)) * M + s % M and value head s / (M * H / G). Scores
 //                    (q . k) * scale, then cap * tanh(score / cap) with a cap. Keys are walked in blocks of 64 aligned
 //                    to absolute positions, wave w takes the blocks with c % 4 == w, the four waves' results are merged
-//                    in wave order: a row's result depends only on its own position and keys
+//                    in wave order: a row's result depends only on its own position and keys. With a window the query
+//                    at p sees keys p + 1 - window .. p and, with keep_first, the keys before keep_first (the blocks
+//                    between them are passed over: their pages may be gone). A sink per head adds exp(sink) to the
+//                    denominator and nothing to the sum
 //   heads_finish     per (row, head): with two maps o = a1 - lambda * a2; optionally o / sqrt(mean(o^2) + eps) * gain;
-//                    optionally times sigmoid(gate) or silu(gate), times a constant; written as the output product's
+//                    optionally times sigmoid(gate) or silu(gate) (a gate per channel or one per head), times a
+//                    constant; written as the output product's
 //                    input (other mixers whose heads end this way use it too)
 //
 // Cache layout of one layer run: keys [page][key slot][page_size][dk], values [page][value head][page_size][dv];

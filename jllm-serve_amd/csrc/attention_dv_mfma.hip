@@ -7,7 +7,9 @@
 // first. Keys are walked in blocks of 64 aligned to absolute positions. Per block the workgroup stages the key slot's
 // K [64][dk] and the value head's V [64][dv] in LDS as they lie in the cache (two buffers: the next block's loads
 // are in flight while this one is multiplied); places outside the tile's visible range are stored as zeros and
-// their table entries are never read.
+// their table entries are never read. With kept first keys (keys before `keep_first` stay visible whatever the window)
+// a tile's blocks are numbered: first the blocks of the kept keys that lie wholly before the window's first block, then
+// the window's; a sink per head adds exp(sink) to the denominator where it is finished (here, or in the merge).
 //
 // Each wave computes the transposed scores S^T[key][row] = K Q^T (v_mfma_f32_32x32x16_bf16, A = K from LDS, B = Q
 // in registers), so a lane owns one query row: maximum and sum are in-lane reductions plus one exchange between the
