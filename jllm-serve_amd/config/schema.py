@@ -237,9 +237,9 @@ class WideAttentionSpec:
     W_g has one row per head and a head's whole output is multiplied by its one number. ``qk_norm`` "head": RMS norm of
     every q head and every k head alone, with one gain vector [dim] for all q heads and one for all k heads (the
     tensors ``<q>.norm`` / ``<k>.norm``). ``window`` > 0: the query at p sees keys p + 1 - window .. p, and, with
-    ``keep_first``, also the keys at positions before ``keep_first`` (which keep their true positions). ``sink``: a
-    learned number per head (tensor ``sink`` [heads]) whose exponential joins the softmax's denominator; it has no key
-    and no value and is not scaled."""
+    ``keep_first``, also the keys at positions before ``keep_first`` (each still at the position it was written at). ``sink``: a
+    learned number per head (tensor ``sink`` [heads]) whose exponential joins the softmax's denominator as it is: nothing
+    is looked up for it, nothing is added to the weighted sum, and the scale does not touch it."""
 
     heads: int
     kv_heads: int
@@ -492,7 +492,7 @@ class LayerSpec:
     mixer_prefix: str = ""  # under the layer's prefix, for mixers whose tensor names are relative to it
     # arrangement "hyper": the stream has ``streams`` copies per row; sublayer q reads u = sum_s in[s] x_s, and all
     # streams are rewritten at once, x_t <- sum_s mix[s, t] x_s + out[t] * sublayer(norm(u)), with the tensors
-    # ``<prefix>.<hyper_names[q]>.in`` [streams], ``.out`` [streams], ``.mix`` [streams, streams] (indexed [from, to])
+    # ``<prefix>.<hyper_names[q]>.in`` [streams], ``.out`` [streams], ``.mix`` [streams, streams] (row: the stream read, column: the stream written)
     streams: int = 1
     hyper_names: Tuple[str, str] = ("hc1", "hc2")
 

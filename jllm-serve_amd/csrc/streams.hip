@@ -7,7 +7,7 @@
 //                  out[t, k, c] = tanh(alpha u[c]) w[c] + b[c] for k < copies, in the output's type (a sublayer's input
 //                  read from the streams; the embedding's norm written once per stream; the final norm of the
 //                  streams' sum over the wanted rows)
-//   streams_write  all streams at once from the old ones: new[r] = sum_s mix[s, r] old[s] + outw[r] y, in place; and,
+//   streams_write  every stream rewritten from the row's previous streams together: new[r] = sum_s mix[s, r] old[s] + outw[r] y, in place; and,
 //                  with next_in, the next sublayer's input from the new streams in the same pass:
 //                  out[t, c] = tanh(alpha sum_r next_in[r] new[r][c]) w[c] + b[c]
 #include <math.h>
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(ST_THREADS) void streams_write_kernel(float* __rest
 #pragma unroll
     for (int s = 0; s < S; ++s) {
       if (s >= streams) break;
-      const float m = mix[s * streams + r];  // mix is indexed [from, to]
+      const float m = mix[s * streams + r];  // row: the stream read, column: the stream written
 #pragma unroll
       for (int i = 0; i < V; ++i) nv.v[i] = fmaf(m, old[s].v[i], nv.v[i]);
     }

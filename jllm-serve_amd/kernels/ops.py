@@ -289,9 +289,9 @@ def dyntanh(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, alpha: to
 
 def streams_write(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out_w: torch.Tensor, *, nxt=None,
                   out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
-    """All streams of every row at once from the old ones, in place on ``x`` fp32 [n, streams x width]:
+    """Every stream of every row rewritten from the row's previous streams together, in place on ``x`` fp32 [n, streams x width]:
     new[r] = sum_s mix[s, r] * old[s] + out_w[r] * y (``y`` fp32 [n, width], a sublayer's output; ``mix`` fp32 [streams,
-    streams] indexed [from, to]). With ``nxt`` = (read [streams], weight, bias, alpha) the next sublayer's input is made
+    streams]: row = the stream read, column = the stream written). With ``nxt`` = (read [streams], weight, bias, alpha) the next sublayer's input is made
     in the same pass from the new streams and returned in ``out_dtype``: tanh(alpha * sum_r read[r] * new[r]) * weight +
     bias."""
     _dev(x, y, mix, out_w)

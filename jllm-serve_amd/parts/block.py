@@ -239,9 +239,9 @@ class StreamReader:
 
 class HyperBlock(Part):
     """Hyper-connections: a row has ``streams`` copies x_1 .. x_s of the residual (fp32, side by side). Sublayer q (the
-    mixer, then the feed-forward) reads u = sum_s in_q[s] x_s, computes y = sublayer(norm_q(u)), and all streams are
-    rewritten at once from the old ones: x_t <- sum_s mix_q[s, t] x_s + out_q[t] * y. The weights are the tensors
-    ``<prefix>.<name>.in`` [streams], ``.out`` [streams] and ``.mix`` [streams, streams] (indexed [from, to]), held in
+    mixer, then the feed-forward) reads u = sum_s in_q[s] x_s, computes y = sublayer(norm_q(u)), and every stream is
+    rewritten from the previous ones together: x_t <- sum_s mix_q[s, t] x_s + out_q[t] * y. The weights are the tensors
+    ``<prefix>.<name>.in`` [streams], ``.out`` [streams] and ``.mix`` [streams, streams] (row: the stream read, column: the stream written), held in
     fp32. Writing the streams and reading the next sublayer's input from them is one launch (``ops.streams_write``), so
     a layer costs two such launches beside its sublayers; the norm must be one that takes no statistics of the row
     (``vectors()``: Dynamic Tanh)."""

@@ -206,7 +206,7 @@ def streams_read(xs: torch.Tensor, w_in: torch.Tensor) -> torch.Tensor:
 
 
 def streams_write(xs: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """All streams at once from the old ones: new[t] = sum_s mix[s, t] old[s] + out[t] y."""
+    """Every stream from the previous streams together: new[t] = sum_s mix[s, t] old[s] + out[t] y."""
     return torch.einsum("sr,stc->rtc", mix, xs) + out[:, None, None] * y[None]
 
 

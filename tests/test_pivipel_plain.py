@@ -212,7 +212,7 @@ def test_plain_sink_is_one_more_term_of_the_denominator_without_a_value():
     for h in range(H):
         sc = torch.einsum("id,jd->ij", q[:, h], k[:, h]) * 0.5
         denom = torch.where(mask, sc.exp(), torch.zeros_like(sc)).sum(dim=1)
-        share = denom / (denom + sink[h].exp())  # the sink is not scaled and counts once
+        share = denom / (denom + sink[h].exp())  # the sink enters as it is, one term
         assert torch.allclose(with_sink[:, h], without[:, h] * share[:, None])
     none = P.attend(q, k, v, 0.5, mask, sink=torch.tensor([-80.0, -80.0], dtype=F64))
     assert torch.allclose(none, without)
@@ -316,7 +316,7 @@ def test_plain_streams(tmp_path):
     mix = torch.randn(3, 3, generator=g, dtype=F64)
     out = torch.randn(3, generator=g, dtype=F64)
     new = P.streams_write(xs, y, mix, out)
-    assert torch.allclose(new[1], mix[0, 1] * xs[0] + mix[1, 1] * xs[1] + mix[2, 1] * xs[2] + out[1] * y), "mix is [from, to]"
+    assert torch.allclose(new[1], mix[0, 1] * xs[0] + mix[1, 1] * xs[1] + mix[2, 1] * xs[2] + out[1] * y), "mix: row = the stream read, column = the stream written"
     assert torch.allclose(P.streams_read(xs, torch.tensor([1.0, 0.0, 2.0], dtype=F64)), xs[0] + 2 * xs[2])
     # identity mixing, every stream read and written with weight 1 / streams resp. 1: the plain residual sum
     folder = pt.write_model(str(tmp_path / "m"), pt.P_D, 7)
