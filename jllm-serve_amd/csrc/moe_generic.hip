@@ -196,23 +196,46 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// A thread owns V neighbouring channels of one row (V = 4 where the width allows 16-byte accesses, else 1): the places
+// and weights of the row's `top` terms, the residual and the shared row are requested before the sum starts, and the
+// terms' loads do not wait for one another. Every output is still one chain of multiply-adds over ascending k.
+template <int V>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
                                                          int top, float weight, const int* __restrict__ place_of,
                                                          const float* __restrict__ weights, const float* __restrict__ shared,
                                                          const float* __restrict__ shared_gate, int ldsg, int overwrite,
                                                          int ld_shared) {
   const int t = blockIdx.x;
+  const int i = (blockIdx.y * 256 + threadIdx.x) * V;
+  if (i >= width) return;
   // a shared expert's rows join the sum, times sigmoid of the row's gate logit where it has one
   const float sg = shared ? (shared_gate ? 1.0f / (1.0f + expf(-shared_gate[(size_t)t * ldsg])) : 1.0f) : 0.f;
-  for (int i = threadIdx.x; i < width; i += 256) {
-    float s = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const size_t row = place_of ? (size_t)place_of[t * top + k] : (size_t)t * top + k;
-      s = weights ? fmaf(weights[(size_t)t * top + k], y[row * width + i], s) : s + y[row * width + i];
+  float r[V], sh[V], s[V];
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    r[c] = overwrite ? 0.f : residual[(size_t)t * width + i + c];
+    sh[c] = shared ? shared[(size_t)t * ld_shared + i + c] : 0.f;
+    s[c] = 0.f;
+  }
+#pragma unroll 4
+  for (int k = 0; k < top; ++k) {
+    const size_t row = place_of ? (size_t)place_of[t * top + k] : (size_t)t * top + k;
+    const float w = weights ? weights[(size_t)t * top + k] : 1.0f;
+    float v[V];
+    if (V == 4) {
+      const float4 q = *(const float4*)(y + row * width + i);
+      v[0] = q.x, v[1 % V] = q.y, v[2 % V] = q.z, v[3 % V] = q.w;
+    } else {
+      v[0] = y[row * width + i];
     }
-    float r = overwrite ? 0.f : residual[(size_t)t * width + i];
-    if (shared) r = fmaf(sg, shared[(size_t)t * ld_shared + i], r);
-    residual[(size_t)t * width + i] = r + weight * s;
+#pragma unroll
+    for (int c = 0; c < V; ++c) s[c] = weights ? fmaf(w, v[c], s[c]) : s[c] + v[c];
+  }
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    float o = r[c];
+    if (shared) o = fmaf(sg, sh[c], o);
+    residual[(size_t)t * width + i + c] = o + weight * s[c];
   }
 }
 
@@ -225,8 +248,15 @@ extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int widt
   if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
   if (shared_gate && !shared) JLLM_FAIL("moe_combine: a gate without the shared rows it weighs");
   if (shared && ld_shared < width) JLLM_FAIL("moe_combine: shared rows %d apart for a width of %d", ld_shared, width);
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg, overwrite,
-                                            ld_shared);
+  const bool vec = width % 4 == 0 && ((uintptr_t)y & 15) == 0;
+  const int per = vec ? 4 : 1;
+  dim3 grid(T, (width + 256 * per - 1) / (256 * per));
+  if (vec)
+    moe_combine_kernel<4><<<grid, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg,
+                                                    overwrite, ld_shared);
+  else
+    moe_combine_kernel<1><<<grid, 256, 0, stream>>>(y, residual, width, top, weight, place_of, weights, shared, shared_gate, ldsg,
+                                                    overwrite, ld_shared);
   JLLM_CHECK_LAUNCH("moe_combine");
   return 0;
 }
